@@ -1,0 +1,472 @@
+// C-ABI entry points: argument validation, the gfx950 launch table, error reporting.
+// Nothing here throws; every failure becomes a negative status plus a thread-local message.
+#include "km_common.h"
+#include "km_launch.h"
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+namespace km {
+
+void host_make_ranges(const float* x1, const float* x2, int64_t num_batch, int64_t n1, int64_t n2,
+                      float cutoff, int bs, bool align, int32_t* start, int32_t* end);
+void host_make_ranges_symmetric(const float* x, int64_t num_batch, int64_t n, float cutoff, int bs,
+                                int32_t* start, int32_t* end);
+void host_transpose_ranges(const int32_t* start, const int32_t* end, int64_t num_batch,
+                           int64_t rows, int x1_size, int x2_size, int bs, int32_t* start_t,
+                           int32_t* end_t);
+
+static thread_local char g_error[512] = "";
+
+static int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+static int fail_hip(const char* what, hipError_t err) {
+    return fail(KM_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(err));
+}
+
+static const long long INT_LIMIT = 2147483647LL;
+
+// Validates the shared part of every device entry point; returns the number of batch items
+// through `num_batches` (0 is legal: nothing to do).
+static int check_common(const char* op, int kernel_type, int batch_rank, const int64_t* batch_sizes,
+                        int64_t m, int64_t n, long long* num_batches) {
+    if (km_num_params(kernel_type) < 0) {
+        return fail(KM_ERR_UNSUPPORTED, "%s: unknown kernel type %d", op, kernel_type);
+    }
+    if (batch_rank < 0 || batch_rank > KM_MAX_BATCH_RANK) {
+        return fail(KM_ERR_UNSUPPORTED, "%s: batch rank %d outside [0, %d]", op, batch_rank,
+                    KM_MAX_BATCH_RANK);
+    }
+    if (batch_rank > 0 && batch_sizes == nullptr) {
+        return fail(KM_ERR_INVALID_ARGUMENT, "%s: batch_sizes is NULL", op);
+    }
+    long long nb = 1;
+    for (int d = 0; d < batch_rank; d++) {
+        if (batch_sizes[d] < 0 || batch_sizes[d] > INT_LIMIT) {
+            return fail(KM_ERR_INVALID_ARGUMENT, "%s: batch size %lld out of range", op,
+                        (long long)batch_sizes[d]);
+        }
+        nb *= batch_sizes[d];
+        if (nb > INT_LIMIT) {
+            return fail(KM_ERR_UNSUPPORTED, "%s: more than 2^31-1 batch items", op);
+        }
+    }
+    if (m < 0 || n < 0 || m > INT_LIMIT - KM_BLOCK_SIZE || n > INT_LIMIT - KM_BLOCK_SIZE) {
+        return fail(KM_ERR_INVALID_ARGUMENT, "%s: matrix size (%lld, %lld) out of range", op,
+                    (long long)m, (long long)n);
+    }
+    *num_batches = nb;
+    return KM_OK;
+}
+
+#define KM_REQUIRE_PTR(op, p)                                                     \
+    do {                                                                          \
+        if ((p) == nullptr) {                                                     \
+            return fail(KM_ERR_INVALID_ARGUMENT, "%s: %s is NULL", (op), #p);    \
+        }                                                                         \
+    } while (0)
+
+// ---------------------------------------------------------------------------------------
+// gfx950 launch table for the forward operator.  256 CUs x 4 SIMDs: aim for at least four
+// wavefronts per SIMD.  Large problems run one wavefront per 128-row block (8 row groups,
+// no cross-wavefront reduction); smaller ones first shrink the rows per wavefront, then
+// let several wavefronts share a row range.
+// ---------------------------------------------------------------------------------------
+static const long long TARGET_WAVES = 4096;
+
+static int make_plan(const MatmulProblem& p, const km_launch_options* opt, MatmulPlan* plan) {
+    int variant = opt ? opt->variant : KM_VARIANT_AUTO;
+    if (variant == KM_VARIANT_AUTO) {
+        variant = KM_VARIANT_MFMA;
+    }
+    if (variant != KM_VARIANT_VALU && variant != KM_VARIANT_MFMA) {
+        return fail(KM_ERR_INVALID_ARGUMENT, "km_matmul: unknown variant %d", variant);
+    }
+    plan->variant = variant;
+    if (variant == KM_VARIANT_VALU) {
+        plan->k_chunk = p.k > 8 ? 16 : (p.k > 4 ? 8 : 4);
+        plan->row_groups = 8;
+        plan->col_splits = 1;
+        return KM_OK;
+    }
+    plan->k_chunk = p.k <= 16 ? 16 : (p.k <= 32 ? 32 : 64);
+    const int G = plan->k_chunk / 16;
+    const long long row_blocks = (p.m + KM_BLOCK_SIZE - 1) / KM_BLOCK_SIZE;
+    const long long base = row_blocks * p.num_batches * ((p.k + plan->k_chunk - 1) / plan->k_chunk);
+
+    int R = 8;
+    if (opt && opt->rows_per_wave != 0) {
+        const int rows = opt->rows_per_wave;
+        if (rows != 16 && rows != 32 && rows != 64 && rows != 128) {
+            return fail(KM_ERR_INVALID_ARGUMENT, "km_matmul: rows_per_wave must be 16, 32, 64 or 128");
+        }
+        R = rows / 16;
+    } else {
+        while (R > 1 && base * (8 / R) < TARGET_WAVES) {
+            R /= 2;
+        }
+    }
+    int S = 1;
+    if (opt && opt->col_splits != 0) {
+        S = opt->col_splits;
+        if (S != 1 && S != 2 && S != 4 && S != 8) {
+            return fail(KM_ERR_INVALID_ARGUMENT, "km_matmul: col_splits must be 1, 2, 4 or 8");
+        }
+    } else {
+        while (S < 8 && base * (8 / R) * S < TARGET_WAVES) {
+            S *= 2;
+        }
+    }
+    // The cross-wavefront reduction buffer (S * R * G KiB) must fit 64 KiB of LDS.
+    while (S > 1 && S * R * G > 64) {
+        S /= 2;
+    }
+    plan->row_groups = R;
+    plan->col_splits = S;
+    return KM_OK;
+}
+
+}  // namespace km
+
+using namespace km;
+
+extern "C" {
+
+const char* km_last_error(void) { return g_error; }
+
+int km_version(void) { return 100; }
+
+int km_num_params(int kernel_type) {
+    switch (kernel_type) {
+        case KM_KERNEL_RBF: return 2;
+        case KM_KERNEL_SPECTRAL: return 3;
+        case KM_KERNEL_LOCALLY_PERIODIC: return 4;
+        default: return -1;
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// Ranges (host).
+// ---------------------------------------------------------------------------------------
+static int check_ranges(const char* op, int64_t num_batch, int64_t n1, int64_t n2, int block_size) {
+    if (block_size <= 0) {
+        return fail(KM_ERR_INVALID_ARGUMENT, "%s: block_size must be positive", op);
+    }
+    if (num_batch < 0 || n1 < 0 || n2 < 0 || n1 > INT_LIMIT - block_size || n2 > INT_LIMIT - block_size) {
+        return fail(KM_ERR_INVALID_ARGUMENT, "%s: sizes out of range", op);
+    }
+    return KM_OK;
+}
+
+int km_make_ranges(const float* x1, const float* x2, int64_t num_batch, int64_t n1, int64_t n2,
+                   float cutoff, int block_size, int align, int32_t* start, int32_t* end) {
+    const char* op = "km_make_ranges";
+    if (int rc = check_ranges(op, num_batch, n1, n2, block_size)) return rc;
+    if (num_batch == 0 || n1 == 0) return KM_OK;
+    KM_REQUIRE_PTR(op, x1);
+    if (n2 > 0) KM_REQUIRE_PTR(op, x2);
+    KM_REQUIRE_PTR(op, start);
+    KM_REQUIRE_PTR(op, end);
+    host_make_ranges(x1, x2, num_batch, n1, n2, cutoff, block_size, align != 0, start, end);
+    return KM_OK;
+}
+
+int km_make_ranges_symmetric(const float* x, int64_t num_batch, int64_t n, float cutoff,
+                             int block_size, int32_t* start, int32_t* end) {
+    const char* op = "km_make_ranges_symmetric";
+    if (int rc = check_ranges(op, num_batch, n, n, block_size)) return rc;
+    if (num_batch == 0 || n == 0) return KM_OK;
+    KM_REQUIRE_PTR(op, x);
+    KM_REQUIRE_PTR(op, start);
+    KM_REQUIRE_PTR(op, end);
+    host_make_ranges_symmetric(x, num_batch, n, cutoff, block_size, start, end);
+    return KM_OK;
+}
+
+int km_transpose_ranges(const int32_t* start, const int32_t* end, int64_t num_batch, int64_t rows,
+                        int x1_size, int x2_size, int block_size, int32_t* start_t, int32_t* end_t) {
+    const char* op = "km_transpose_ranges";
+    if (block_size <= 0) return fail(KM_ERR_INVALID_ARGUMENT, "%s: block_size must be positive", op);
+    if (num_batch < 0 || rows < 0 || x1_size < 0 || x2_size < 0) {
+        return fail(KM_ERR_INVALID_ARGUMENT, "%s: sizes out of range", op);
+    }
+    if (rows != ((int64_t)x1_size + block_size - 1) / block_size) {
+        return fail(KM_ERR_INVALID_ARGUMENT, "%s: rows (%lld) does not match ceil(x1_size / block_size)",
+                    op, (long long)rows);
+    }
+    if (num_batch == 0 || x2_size == 0) return KM_OK;
+    if (rows > 0) {
+        KM_REQUIRE_PTR(op, start);
+        KM_REQUIRE_PTR(op, end);
+    }
+    KM_REQUIRE_PTR(op, start_t);
+    KM_REQUIRE_PTR(op, end_t);
+    host_transpose_ranges(start, end, num_batch, rows, x1_size, x2_size, block_size, start_t, end_t);
+    return KM_OK;
+}
+
+// ---------------------------------------------------------------------------------------
+// Ranges (device).
+// ---------------------------------------------------------------------------------------
+int km_make_ranges_device(const float* x1, const float* x2, int64_t num_batch, int64_t n1,
+                          int64_t n2, float cutoff, int block_size, int align, int32_t* start,
+                          int32_t* end, void* stream) {
+    const char* op = "km_make_ranges_device";
+    if (int rc = check_ranges(op, num_batch, n1, n2, block_size)) return rc;
+    if (num_batch == 0 || n1 == 0) return KM_OK;
+    KM_REQUIRE_PTR(op, x1);
+    if (n2 > 0) KM_REQUIRE_PTR(op, x2);
+    KM_REQUIRE_PTR(op, start);
+    KM_REQUIRE_PTR(op, end);
+    hipError_t err = launch_make_ranges(x1, x2, num_batch, n1, n2, cutoff, block_size, align, start,
+                                        end, (hipStream_t)stream);
+    return err == hipSuccess ? KM_OK : fail_hip(op, err);
+}
+
+int km_make_ranges_symmetric_device(const float* x, int64_t num_batch, int64_t n, float cutoff,
+                                    int block_size, int32_t* start, int32_t* end, void* stream) {
+    const char* op = "km_make_ranges_symmetric_device";
+    if (int rc = check_ranges(op, num_batch, n, n, block_size)) return rc;
+    if (num_batch == 0 || n == 0) return KM_OK;
+    KM_REQUIRE_PTR(op, x);
+    KM_REQUIRE_PTR(op, start);
+    KM_REQUIRE_PTR(op, end);
+    hipError_t err = launch_make_ranges_symmetric(x, num_batch, n, cutoff, block_size, start, end,
+                                                  (hipStream_t)stream);
+    return err == hipSuccess ? KM_OK : fail_hip(op, err);
+}
+
+// ---------------------------------------------------------------------------------------
+// matmul
+// ---------------------------------------------------------------------------------------
+int km_matmul(int kernel_type, int batch_rank, const int64_t* batch_sizes, int64_t m, int64_t n,
+              int64_t k, const float* x1, const int64_t* x1_strides, const float* x2,
+              const int64_t* x2_strides, const float* rhs, const int64_t* rhs_strides,
+              const float* params, const int64_t* params_strides, const int32_t* start,
+              const int64_t* start_strides, const int32_t* end, const int64_t* end_strides,
+              float* out, const km_launch_options* options, void* stream) {
+    const char* op = "km_matmul";
+    long long nb = 0;
+    if (int rc = check_common(op, kernel_type, batch_rank, batch_sizes, m, n, &nb)) return rc;
+    if (k < 0 || k > INT_LIMIT) return fail(KM_ERR_INVALID_ARGUMENT, "%s: k out of range", op);
+    if ((long long)m * k > INT_LIMIT * 64LL) {
+        return fail(KM_ERR_UNSUPPORTED, "%s: m * k too large", op);
+    }
+    if (nb == 0 || m == 0 || k == 0) return KM_OK;
+    KM_REQUIRE_PTR(op, x1);
+    KM_REQUIRE_PTR(op, x1_strides);
+    KM_REQUIRE_PTR(op, x2_strides);
+    KM_REQUIRE_PTR(op, rhs_strides);
+    KM_REQUIRE_PTR(op, params);
+    KM_REQUIRE_PTR(op, params_strides);
+    KM_REQUIRE_PTR(op, start);
+    KM_REQUIRE_PTR(op, start_strides);
+    KM_REQUIRE_PTR(op, end);
+    KM_REQUIRE_PTR(op, end_strides);
+    KM_REQUIRE_PTR(op, out);
+    if (n > 0) {
+        KM_REQUIRE_PTR(op, x2);
+        KM_REQUIRE_PTR(op, rhs);
+    }
+
+    MatmulProblem p;
+    p.kernel_type = kernel_type;
+    p.batch_rank = batch_rank;
+    p.batch_sizes = batch_sizes;
+    p.num_batches = nb;
+    p.m = m;
+    p.n = n;
+    p.k = k;
+    p.x1 = x1;
+    p.x1_strides = x1_strides;
+    p.x2 = x2;
+    p.x2_strides = x2_strides;
+    p.rhs = rhs;
+    p.rhs_strides = rhs_strides;
+    p.params = params;
+    p.params_strides = params_strides;
+    p.start = start;
+    p.start_strides = start_strides;
+    p.end = end;
+    p.end_strides = end_strides;
+    p.out = out;
+
+    MatmulPlan plan;
+    if (int rc = make_plan(p, options, &plan)) return rc;
+    hipError_t err = launch_matmul(p, plan, (hipStream_t)stream);
+    return err == hipSuccess ? KM_OK : fail_hip(op, err);
+}
+
+// ---------------------------------------------------------------------------------------
+// param_grad (matmul_bwd and bilinear_derivative)
+// ---------------------------------------------------------------------------------------
+size_t km_param_grad_workspace_size(int kernel_type, int batch_rank, const int64_t* batch_sizes,
+                                    int64_t m, int64_t n, int64_t c) {
+    (void)c;
+    long long nb = 0;
+    if (check_common("km_param_grad_workspace_size", kernel_type, batch_rank, batch_sizes, m, n, &nb)) {
+        return 0;
+    }
+    if (nb == 0 || m == 0) return 0;
+    return (size_t)nb * (size_t)param_grad_partials_per_batch(m, nb) * KM_MAX_PARAMS * sizeof(float);
+}
+
+int km_param_grad(int kernel_type, int batch_rank, const int64_t* batch_sizes, int64_t m,
+                  int64_t n, int64_t c, const float* x1, const int64_t* x1_strides,
+                  const float* x2, const int64_t* x2_strides, const float* left,
+                  const int64_t* left_strides, const float* right, const int64_t* right_strides,
+                  const float* params, const int64_t* params_strides, const int32_t* start,
+                  const int64_t* start_strides, const int32_t* end, const int64_t* end_strides,
+                  float* grad, void* workspace, size_t workspace_bytes, void* stream) {
+    const char* op = "km_param_grad";
+    long long nb = 0;
+    if (int rc = check_common(op, kernel_type, batch_rank, batch_sizes, m, n, &nb)) return rc;
+    if (c < 0 || c > INT_LIMIT) return fail(KM_ERR_INVALID_ARGUMENT, "%s: c out of range", op);
+    if (nb == 0) return KM_OK;
+    KM_REQUIRE_PTR(op, grad);
+    KM_REQUIRE_PTR(op, params);
+    KM_REQUIRE_PTR(op, params_strides);
+    KM_REQUIRE_PTR(op, x1_strides);
+    KM_REQUIRE_PTR(op, x2_strides);
+    KM_REQUIRE_PTR(op, left_strides);
+    KM_REQUIRE_PTR(op, right_strides);
+    KM_REQUIRE_PTR(op, start_strides);
+    KM_REQUIRE_PTR(op, end_strides);
+    if (m > 0) {
+        KM_REQUIRE_PTR(op, x1);
+        KM_REQUIRE_PTR(op, start);
+        KM_REQUIRE_PTR(op, end);
+        if (c > 0) KM_REQUIRE_PTR(op, left);
+    }
+    if (n > 0) {
+        KM_REQUIRE_PTR(op, x2);
+        if (c > 0) KM_REQUIRE_PTR(op, right);
+    }
+    const size_t need = km_param_grad_workspace_size(kernel_type, batch_rank, batch_sizes, m, n, c);
+    if (need > 0 && (workspace == nullptr || workspace_bytes < need)) {
+        return fail(KM_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", op, need,
+                    workspace ? workspace_bytes : (size_t)0);
+    }
+
+    ParamGradProblem p;
+    p.kernel_type = kernel_type;
+    p.batch_rank = batch_rank;
+    p.batch_sizes = batch_sizes;
+    p.num_batches = nb;
+    p.m = m;
+    p.n = n;
+    p.c = c;
+    p.x1 = x1;
+    p.x1_strides = x1_strides;
+    p.x2 = x2;
+    p.x2_strides = x2_strides;
+    p.left = left;
+    p.left_strides = left_strides;
+    p.right = right;
+    p.right_strides = right_strides;
+    p.params = params;
+    p.params_strides = params_strides;
+    p.start = start;
+    p.start_strides = start_strides;
+    p.end = end;
+    p.end_strides = end_strides;
+    p.grad = grad;
+    p.workspace = workspace;
+    hipError_t err = launch_param_grad(p, (hipStream_t)stream);
+    return err == hipSuccess ? KM_OK : fail_hip(op, err);
+}
+
+// ---------------------------------------------------------------------------------------
+// index
+// ---------------------------------------------------------------------------------------
+int km_index(int kernel_type, int batch_rank, const int64_t* batch_sizes, int64_t m, int64_t n,
+             const float* x1, const int64_t* x1_strides, const float* x2,
+             const int64_t* x2_strides, const float* params, const int64_t* params_strides,
+             const int32_t* start, const int64_t* start_strides, const int32_t* end,
+             const int64_t* end_strides, int index_rank, const int64_t* index_sizes,
+             const int32_t* const* batch_index, const int64_t* const* batch_index_strides,
+             const int32_t* row_index, const int64_t* row_index_strides,
+             const int32_t* col_index, const int64_t* col_index_strides, float* out,
+             void* stream) {
+    const char* op = "km_index";
+    long long nb = 0;
+    if (int rc = check_common(op, kernel_type, batch_rank, batch_sizes, m, n, &nb)) return rc;
+    if (index_rank < 1 || index_rank > KM_MAX_BATCH_RANK + 1) {
+        return fail(KM_ERR_UNSUPPORTED, "%s: index rank %d outside [1, %d]", op, index_rank,
+                    KM_MAX_BATCH_RANK + 1);
+    }
+    KM_REQUIRE_PTR(op, index_sizes);
+    long long total = 1;
+    for (int d = 0; d < index_rank; d++) {
+        if (index_sizes[d] < 0) return fail(KM_ERR_INVALID_ARGUMENT, "%s: negative index size", op);
+        total *= index_sizes[d];
+        if (total > INT_LIMIT * 256LL) return fail(KM_ERR_UNSUPPORTED, "%s: too many index entries", op);
+    }
+    if (total == 0) return KM_OK;
+    KM_REQUIRE_PTR(op, out);
+    KM_REQUIRE_PTR(op, row_index);
+    KM_REQUIRE_PTR(op, row_index_strides);
+    KM_REQUIRE_PTR(op, col_index);
+    KM_REQUIRE_PTR(op, col_index_strides);
+    KM_REQUIRE_PTR(op, x1_strides);
+    KM_REQUIRE_PTR(op, x2_strides);
+    KM_REQUIRE_PTR(op, params_strides);
+    KM_REQUIRE_PTR(op, start_strides);
+    KM_REQUIRE_PTR(op, end_strides);
+    if (batch_rank > 0) {
+        KM_REQUIRE_PTR(op, batch_index);
+        KM_REQUIRE_PTR(op, batch_index_strides);
+        for (int d = 0; d < batch_rank; d++) {
+            if (batch_index[d] == nullptr || batch_index_strides[d] == nullptr) {
+                return fail(KM_ERR_INVALID_ARGUMENT, "%s: batch_index[%d] is NULL", op, d);
+            }
+        }
+    }
+    // With an empty matrix no entry can be inside it; the kernel then only writes zeros and
+    // never dereferences the matrix inputs.
+    const bool empty = nb == 0 || m == 0 || n == 0;
+    if (!empty) {
+        KM_REQUIRE_PTR(op, x1);
+        KM_REQUIRE_PTR(op, x2);
+        KM_REQUIRE_PTR(op, params);
+        KM_REQUIRE_PTR(op, start);
+        KM_REQUIRE_PTR(op, end);
+    }
+
+    IndexProblem p;
+    p.kernel_type = kernel_type;
+    p.batch_rank = batch_rank;
+    p.batch_sizes = batch_sizes;
+    p.m = empty ? 0 : m;
+    p.n = empty ? 0 : n;
+    p.x1 = x1;
+    p.x1_strides = x1_strides;
+    p.x2 = x2;
+    p.x2_strides = x2_strides;
+    p.params = params;
+    p.params_strides = params_strides;
+    p.start = start;
+    p.start_strides = start_strides;
+    p.end = end;
+    p.end_strides = end_strides;
+    p.index_rank = index_rank;
+    p.index_sizes = index_sizes;
+    p.batch_index = batch_index;
+    p.batch_index_strides = batch_index_strides;
+    p.row_index = row_index;
+    p.row_index_strides = row_index_strides;
+    p.col_index = col_index;
+    p.col_index_strides = col_index_strides;
+    p.out = out;
+    hipError_t err = launch_index(p, (hipStream_t)stream);
+    return err == hipSuccess ? KM_OK : fail_hip(op, err);
+}
+
+}  // extern "C"

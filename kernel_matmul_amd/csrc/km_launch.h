@@ -1,0 +1,106 @@
+// Host-side problem descriptions shared by the C-ABI layer and the kernel launchers.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace km {
+
+enum { KM_VARIANT_AUTO = 0, KM_VARIANT_VALU = 1, KM_VARIANT_MFMA = 2 };
+
+struct MatmulProblem {
+    int kernel_type;
+    int batch_rank;
+    const int64_t* batch_sizes;
+    long long num_batches;
+    int64_t m, n, k;
+    const float* x1;
+    const int64_t* x1_strides;
+    const float* x2;
+    const int64_t* x2_strides;
+    const float* rhs;
+    const int64_t* rhs_strides;
+    const float* params;
+    const int64_t* params_strides;
+    const int32_t* start;
+    const int64_t* start_strides;
+    const int32_t* end;
+    const int64_t* end_strides;
+    float* out;
+};
+
+// Which ahead-of-time instantiation runs and with what decomposition.
+struct MatmulPlan {
+    int variant;     // KM_VARIANT_VALU or KM_VARIANT_MFMA
+    int k_chunk;     // rhs columns handled per workgroup (MFMA: 16/32/64, VALU: 4/8/16)
+    int row_groups;  // MFMA: groups of 16 rows per wavefront (1, 2, 4, 8)
+    int col_splits;  // MFMA: wavefronts per workgroup sharing one column range (1, 2, 4, 8)
+};
+
+hipError_t launch_matmul(const MatmulProblem& p, const MatmulPlan& plan, hipStream_t stream);
+
+struct ParamGradProblem {
+    int kernel_type;
+    int batch_rank;
+    const int64_t* batch_sizes;
+    long long num_batches;
+    int64_t m, n, c;
+    const float* x1;
+    const int64_t* x1_strides;
+    const float* x2;
+    const int64_t* x2_strides;
+    const float* left;
+    const int64_t* left_strides;
+    const float* right;
+    const int64_t* right_strides;
+    const float* params;
+    const int64_t* params_strides;
+    const int32_t* start;
+    const int64_t* start_strides;
+    const int32_t* end;
+    const int64_t* end_strides;
+    float* grad;
+    void* workspace;
+};
+
+// Partial sums written by the first pass: one row of KM_MAX_PARAMS floats per wavefront.
+long long param_grad_partials_per_batch(int64_t m, long long num_batches);
+hipError_t launch_param_grad(const ParamGradProblem& p, hipStream_t stream);
+
+struct IndexProblem {
+    int kernel_type;
+    int batch_rank;
+    const int64_t* batch_sizes;
+    int64_t m, n;
+    const float* x1;
+    const int64_t* x1_strides;
+    const float* x2;
+    const int64_t* x2_strides;
+    const float* params;
+    const int64_t* params_strides;
+    const int32_t* start;
+    const int64_t* start_strides;
+    const int32_t* end;
+    const int64_t* end_strides;
+    int index_rank;
+    const int64_t* index_sizes;
+    const int32_t* const* batch_index;
+    const int64_t* const* batch_index_strides;
+    const int32_t* row_index;
+    const int64_t* row_index_strides;
+    const int32_t* col_index;
+    const int64_t* col_index_strides;
+    float* out;
+};
+
+hipError_t launch_index(const IndexProblem& p, hipStream_t stream);
+
+hipError_t launch_make_ranges(const float* x1, const float* x2, int64_t num_batch, int64_t n1,
+                              int64_t n2, float cutoff, int block_size, int align, int32_t* start,
+                              int32_t* end, hipStream_t stream);
+hipError_t launch_make_ranges_symmetric(const float* x, int64_t num_batch, int64_t n, float cutoff,
+                                        int block_size, int32_t* start, int32_t* end,
+                                        hipStream_t stream);
+
+}  // namespace km

@@ -1,0 +1,397 @@
+// Hyper-parameter gradient of sum_{(i,j) in mask} C[i,j] K[i,j] with C = left @ right^T.
+// Serves the reference operators matmul_bwd (left = out_grad, right = rhs;
+// native/matmul_bwd/matmul_bwd.cu:12-221) and bilinear_derivative
+// (native/bilinear_derivative/bilinear_derivative.cu:12-183), which compute the same sum.
+//
+// Pass 1 (param_grad_partial): a wavefront owns 128 rows and a share of the row block's
+// column range.  Per 16-column chunk and 16-row group the coefficient tile C (16x16) is
+// formed on the matrix pipe from left/right (v_mfma_f32_16x16x4_f32 over the vector
+// columns); its D layout gives each lane 4 (row, col) pairs, for which the lane evaluates
+// the kernel derivatives and accumulates per-lane sums.  The sums are combined across the
+// wavefront with DPP/permute shuffles and written as one partial row per wavefront.
+// Pass 2 (param_grad_reduce): one workgroup per batch item adds the partial rows in a
+// fixed order in fp64 and applies the chain rule back to the user parameters
+// (native/common/kernel_function.cuh:221-251).  No atomics: results are reproducible.
+#include "km_common.h"
+#include "km_launch.h"
+
+namespace km {
+
+struct GradArgs {
+    BatchShape batch;
+    long long num_batches;
+    long long total_items;  // row blocks * col splits * batches
+    long long items_per_xcd;
+    int m, n, c;
+    int col_splits;
+    const float* x1;
+    const float* x2;
+    const float* left;
+    const float* right;
+    const float* params;
+    const int* start;
+    const int* end;
+    float* partials;  // [num_batches][row_blocks * col_splits][KM_MAX_PARAMS]
+    BatchStrides x1_bs, x2_bs, left_bs, right_bs, params_bs, start_bs, end_bs;
+    long long x1_s, x2_s, left_s0, left_s1, right_s0, right_s1, params_s, start_s, end_s;
+};
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        v += __shfl_xor(v, off, 64);
+    }
+    return v;
+}
+
+// Accumulates the per-pair derivative terms.  acc[] meaning per kernel type:
+//   rbf      : acc0 = sum C E u^2,  acc1 = sum C E
+//   spectral : acc0 = sum C E cos u^2,  acc1 = sum C E sin d,  acc2 = sum C E cos
+//   loc.per. : acc0 = sum C E u^2,  acc1 = sum C E sin^2,  acc2 = sum C E sin cos d,  acc3 = sum C E
+// with E the kernel value without sigma.
+template <int KT>
+__device__ __forceinline__ void accumulate_pair(float x1, float x2, float coeff,
+                                                const KernelConsts& kc, float (&acc)[KM_MAX_PARAMS]) {
+    const float d = x1 - x2;
+    const float u = d * kc.s;
+    const float uu = u * u;
+    if (KT == KM_KERNEL_RBF) {
+        const float w = coeff * __builtin_amdgcn_exp2f(-uu);
+        acc[0] = __builtin_fmaf(w, uu, acc[0]);
+        acc[1] += w;
+    } else if (KT == KM_KERNEL_SPECTRAL) {
+        const float ph = d * kc.f;
+        const float w = coeff * __builtin_amdgcn_exp2f(-uu);
+        const float wc = w * __builtin_amdgcn_cosf(ph);
+        const float ws = w * __builtin_amdgcn_sinf(ph);
+        acc[0] = __builtin_fmaf(wc, uu, acc[0]);
+        acc[1] = __builtin_fmaf(ws, d, acc[1]);
+        acc[2] += wc;
+    } else {
+        const float ph = d * kc.f;
+        const float sn = __builtin_amdgcn_sinf(ph);
+        const float cs = __builtin_amdgcn_cosf(ph);
+        const float q = sn * sn;
+        const float w = coeff * __builtin_amdgcn_exp2f(__builtin_fmaf(-kc.cl, q, -uu));
+        acc[0] = __builtin_fmaf(w, uu, acc[0]);
+        acc[1] = __builtin_fmaf(w, q, acc[1]);
+        acc[2] = __builtin_fmaf(w * (sn * cs), d, acc[2]);
+        acc[3] += w;
+    }
+}
+
+// TL > 0: the vector width c is at most 4*TL and the left operand stays in registers.
+// TL == 0: any c; the left operand is re-read (from L1/L2) for every column chunk.
+template <int KT, int TL>
+__global__ void __launch_bounds__(64) param_grad_partial(const GradArgs a) {
+    constexpr int R = 8;
+    const int lane = threadIdx.x;
+    const int li = lane & 15;
+    const int kk = lane >> 4;
+
+    const long long item = xcd_item(blockIdx.x, a.items_per_xcd);
+    if (item >= a.total_items) {
+        return;
+    }
+    const long long b = item % a.num_batches;
+    const long long rest = item / a.num_batches;
+    const int split = (int)(rest % a.col_splits);
+    const int row_block = (int)(rest / a.col_splits);
+    const int row0 = row_block * KM_BLOCK_SIZE;
+
+    int bidx[KM_MAX_BATCH_RANK];
+    batch_multi_index(a.batch, b, bidx);
+    const float* __restrict__ x1 = a.x1 + batch_offset(a.batch, a.x1_bs, bidx);
+    const float* __restrict__ x2 = a.x2 + batch_offset(a.batch, a.x2_bs, bidx);
+    const float* __restrict__ left = a.left + batch_offset(a.batch, a.left_bs, bidx);
+    const float* __restrict__ right = a.right + batch_offset(a.batch, a.right_bs, bidx);
+    const float* __restrict__ params = a.params + batch_offset(a.batch, a.params_bs, bidx);
+    int range_start = a.start[batch_offset(a.batch, a.start_bs, bidx) + row_block * a.start_s];
+    int range_end = a.end[batch_offset(a.batch, a.end_bs, bidx) + row_block * a.end_s];
+    range_start = max(range_start, 0);
+    range_end = min(range_end, a.n);
+
+    const KernelConsts kc = make_consts<KT>(params, a.params_s, false);
+
+    // Column share of this wavefront, in whole chunks of 16 columns.
+    const int width = max(range_end - range_start, 0);
+    const int per_split = ((width + a.col_splits - 1) / a.col_splits + 15) & ~15;
+    const int col_begin = range_start + split * per_split;
+    const int col_end = min(range_end, col_begin + per_split);
+
+    // x1 for the 4 rows per row group this lane owns in the D layout.
+    float x1q[R][4];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            const int row = min(row0 + 16 * r + 4 * kk + v, a.m - 1);
+            x1q[r][v] = x1[(long long)row * a.x1_s];
+        }
+    }
+
+    // Left operand (A layout): row = row0 + 16 r + li, vector column = 4 t + kk.
+    constexpr int TLR = TL > 0 ? TL : 1;
+    float lreg[R][TLR];
+    if (TL > 0) {
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int row = row0 + 16 * r + li;
+#pragma unroll
+            for (int t = 0; t < TLR; t++) {
+                const int cc = 4 * t + kk;
+                lreg[r][t] = (row < a.m && cc < a.c)
+                                 ? left[(long long)row * a.left_s0 + (long long)cc * a.left_s1]
+                                 : 0.0f;
+            }
+        }
+    }
+
+    float acc[KM_MAX_PARAMS] = {0.0f, 0.0f, 0.0f, 0.0f};
+
+    for (int n0 = col_begin; n0 < col_end; n0 += 16) {
+        const int col = n0 + li;
+        const bool col_ok = col < col_end;
+        const int col_c = min(col, col_end - 1);
+        const float x2v = x2[(long long)col_c * a.x2_s];
+
+        float4v coef[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            coef[r] = (float4v){0.0f, 0.0f, 0.0f, 0.0f};
+        }
+
+        if (TL > 0) {
+#pragma unroll
+            for (int t = 0; t < TLR; t++) {
+                const int cc = 4 * t + kk;
+                const float rv = (col_ok && cc < a.c)
+                                     ? right[(long long)col_c * a.right_s0 + (long long)cc * a.right_s1]
+                                     : 0.0f;
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    coef[r] = __builtin_amdgcn_mfma_f32_16x16x4f32(lreg[r][t], rv, coef[r], 0, 0, 0);
+                }
+            }
+        } else {
+            for (int c0 = 0; c0 < a.c; c0 += 4) {
+                const int cc = c0 + kk;
+                const float rv = (col_ok && cc < a.c)
+                                     ? right[(long long)col_c * a.right_s0 + (long long)cc * a.right_s1]
+                                     : 0.0f;
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    const int row = row0 + 16 * r + li;
+                    const float lv = (row < a.m && cc < a.c)
+                                         ? left[(long long)row * a.left_s0 + (long long)cc * a.left_s1]
+                                         : 0.0f;
+                    coef[r] = __builtin_amdgcn_mfma_f32_16x16x4f32(lv, rv, coef[r], 0, 0, 0);
+                }
+            }
+        }
+
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                accumulate_pair<KT>(x1q[r][v], x2v, coef[r][v], kc, acc);
+            }
+        }
+    }
+
+    const long long partial_rows = a.total_items / a.num_batches;
+    float* __restrict__ prow = a.partials + (b * partial_rows + rest) * KM_MAX_PARAMS;
+#pragma unroll
+    for (int p = 0; p < KM_MAX_PARAMS; p++) {
+        const float total = wave_sum(acc[p]);
+        if (lane == 0) {
+            prow[p] = total;
+        }
+    }
+}
+
+struct ReduceArgs {
+    BatchShape batch;
+    long long partial_rows;
+    const float* partials;
+    const float* params;
+    BatchStrides params_bs;
+    long long params_s;
+    float* grad;  // [num_batches][P]
+};
+
+template <int KT>
+__global__ void __launch_bounds__(256) param_grad_reduce(const ReduceArgs a) {
+    constexpr int P = KernelTraits<KT>::P;
+    __shared__ double sh[KM_MAX_PARAMS][256];
+    const long long b = blockIdx.x;
+    const float* __restrict__ rows = a.partials + b * a.partial_rows * KM_MAX_PARAMS;
+
+    double sum[KM_MAX_PARAMS] = {0.0, 0.0, 0.0, 0.0};
+    for (long long i = threadIdx.x; i < a.partial_rows; i += 256) {
+#pragma unroll
+        for (int p = 0; p < KM_MAX_PARAMS; p++) {
+            sum[p] += (double)rows[i * KM_MAX_PARAMS + p];
+        }
+    }
+#pragma unroll
+    for (int p = 0; p < KM_MAX_PARAMS; p++) {
+        sh[p][threadIdx.x] = sum[p];
+    }
+    __syncthreads();
+    for (int half = 128; half >= 1; half >>= 1) {
+        if ((int)threadIdx.x < half) {
+#pragma unroll
+            for (int p = 0; p < KM_MAX_PARAMS; p++) {
+                sh[p][threadIdx.x] += sh[p][threadIdx.x + half];
+            }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x != 0) {
+        return;
+    }
+
+    int bidx[KM_MAX_BATCH_RANK];
+    batch_multi_index(a.batch, b, bidx);
+    const float* __restrict__ params = a.params + batch_offset(a.batch, a.params_bs, bidx);
+    float* __restrict__ g = a.grad + b * P;
+    const double s0 = sh[0][0], s1 = sh[1][0], s2 = sh[2][0], s3 = sh[3][0];
+    const double l = (double)params[0];
+    const double sigma = (double)params[KernelTraits<KT>::SIGMA * a.params_s];
+    if (KT == KM_KERNEL_RBF) {
+        g[0] = (float)(sigma * s0 * KM_2LN2 / l);
+        g[1] = (float)s1;
+    } else if (KT == KM_KERNEL_SPECTRAL) {
+        g[0] = (float)(sigma * s0 * KM_2LN2 / l);
+        g[1] = (float)(-2.0 * KM_PI * sigma * s1);
+        g[2] = (float)s2;
+    } else {
+        const double lp = (double)params[a.params_s];
+        const double period = (double)params[2 * a.params_s];
+        g[0] = (float)(sigma * s0 * KM_2LN2 / l);
+        g[1] = (float)(2.0 * sigma * s1 / (lp * lp));
+        g[2] = (float)(4.0 * KM_PI * sigma * s2 / (lp * period * period));
+        g[3] = (float)s3;
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// Host dispatch.
+// ---------------------------------------------------------------------------------------
+static int grad_col_splits(int64_t m, long long num_batches) {
+    // Enough wavefronts to populate the 1024 SIMDs of the device several times over when the
+    // row-block count alone does not.
+    const long long row_blocks = (m + KM_BLOCK_SIZE - 1) / KM_BLOCK_SIZE;
+    const long long base = row_blocks * num_batches;
+    if (base <= 0) {
+        return 1;
+    }
+    long long s = (4096 + base - 1) / base;
+    if (s < 1) s = 1;
+    if (s > 16) s = 16;
+    return (int)s;
+}
+
+long long param_grad_partials_per_batch(int64_t m, long long num_batches) {
+    const long long row_blocks = (m + KM_BLOCK_SIZE - 1) / KM_BLOCK_SIZE;
+    return row_blocks * grad_col_splits(m, num_batches);
+}
+
+static void fill_strides(BatchStrides& dst, const int64_t* strides, int rank) {
+    for (int d = 0; d < KM_MAX_BATCH_RANK; d++) {
+        dst.s[d] = d < rank ? strides[d] : 0;
+    }
+}
+
+template <int KT>
+static hipError_t launch_partial(const GradArgs& a, unsigned grid_x, hipStream_t stream) {
+    if (a.c <= 4) {
+        hipLaunchKernelGGL((param_grad_partial<KT, 1>), dim3(grid_x), dim3(64), 0, stream, a);
+    } else if (a.c <= 8) {
+        hipLaunchKernelGGL((param_grad_partial<KT, 2>), dim3(grid_x), dim3(64), 0, stream, a);
+    } else if (a.c <= 16) {
+        hipLaunchKernelGGL((param_grad_partial<KT, 4>), dim3(grid_x), dim3(64), 0, stream, a);
+    } else {
+        hipLaunchKernelGGL((param_grad_partial<KT, 0>), dim3(grid_x), dim3(64), 0, stream, a);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_param_grad(const ParamGradProblem& p, hipStream_t stream) {
+    GradArgs a;
+    const int r = p.batch_rank;
+    a.batch.rank = r;
+    for (int d = 0; d < KM_MAX_BATCH_RANK; d++) {
+        a.batch.sizes[d] = d < r ? (int)p.batch_sizes[d] : 1;
+    }
+    a.num_batches = p.num_batches;
+    a.m = (int)p.m;
+    a.n = (int)p.n;
+    a.c = (int)p.c;
+    a.col_splits = grad_col_splits(p.m, p.num_batches);
+    const long long row_blocks = (p.m + KM_BLOCK_SIZE - 1) / KM_BLOCK_SIZE;
+    a.total_items = row_blocks * a.col_splits * p.num_batches;
+    a.items_per_xcd = (a.total_items + KM_NUM_XCD - 1) / KM_NUM_XCD;
+    a.x1 = p.x1;
+    a.x2 = p.x2;
+    a.left = p.left;
+    a.right = p.right;
+    a.params = p.params;
+    a.start = p.start;
+    a.end = p.end;
+    a.partials = (float*)p.workspace;
+    fill_strides(a.x1_bs, p.x1_strides, r);
+    fill_strides(a.x2_bs, p.x2_strides, r);
+    fill_strides(a.left_bs, p.left_strides, r);
+    fill_strides(a.right_bs, p.right_strides, r);
+    fill_strides(a.params_bs, p.params_strides, r);
+    fill_strides(a.start_bs, p.start_strides, r);
+    fill_strides(a.end_bs, p.end_strides, r);
+    a.x1_s = p.x1_strides[r];
+    a.x2_s = p.x2_strides[r];
+    a.left_s0 = p.left_strides[r];
+    a.left_s1 = p.left_strides[r + 1];
+    a.right_s0 = p.right_strides[r];
+    a.right_s1 = p.right_strides[r + 1];
+    a.params_s = p.params_strides[r];
+    a.start_s = p.start_strides[r];
+    a.end_s = p.end_strides[r];
+
+    const unsigned grid_x = (unsigned)(a.items_per_xcd * KM_NUM_XCD);
+    if (grid_x > 0) {  // no rows: the reduce pass alone writes the zero gradient
+        hipError_t err;
+        switch (p.kernel_type) {
+            case KM_KERNEL_RBF: err = launch_partial<KM_KERNEL_RBF>(a, grid_x, stream); break;
+            case KM_KERNEL_SPECTRAL: err = launch_partial<KM_KERNEL_SPECTRAL>(a, grid_x, stream); break;
+            default: err = launch_partial<KM_KERNEL_LOCALLY_PERIODIC>(a, grid_x, stream); break;
+        }
+        if (err != hipSuccess) {
+            return err;
+        }
+    }
+
+    ReduceArgs ra;
+    ra.batch = a.batch;
+    ra.partial_rows = row_blocks * a.col_splits;
+    ra.partials = a.partials;
+    ra.params = p.params;
+    ra.params_bs = a.params_bs;
+    ra.params_s = a.params_s;
+    ra.grad = p.grad;
+    const unsigned rgrid = (unsigned)p.num_batches;
+    switch (p.kernel_type) {
+        case KM_KERNEL_RBF:
+            hipLaunchKernelGGL((param_grad_reduce<KM_KERNEL_RBF>), dim3(rgrid), dim3(256), 0, stream, ra);
+            break;
+        case KM_KERNEL_SPECTRAL:
+            hipLaunchKernelGGL((param_grad_reduce<KM_KERNEL_SPECTRAL>), dim3(rgrid), dim3(256), 0, stream, ra);
+            break;
+        default:
+            hipLaunchKernelGGL((param_grad_reduce<KM_KERNEL_LOCALLY_PERIODIC>), dim3(rgrid), dim3(256), 0, stream, ra);
+            break;
+    }
+    return hipGetLastError();
+}
+
+}  // namespace km

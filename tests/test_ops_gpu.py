@@ -1,0 +1,121 @@
+"""GPU parity of the four device operators against the float64 oracle, through the same
+``load_native(name, defines).call(*args)`` path the reference's tests use
+(tests/native/test_matmul.py, test_matmul_bwd.py, test_bilinear_derivative.py, test_index.py).
+
+Tolerances: forward/index rtol 1e-4 / atol 1e-5 (tighter than the reference's atol 2e-4);
+gradients rtol 1e-4 / atol 1e-5 relative to the gradient scale (reference: 2e-3)."""
+import numpy as np
+import pytest
+import torch
+
+from kernel_matmul_amd.compile import load_native
+from kernel_matmul_amd.configurations import (
+    BilinearDerivativeConfiguration,
+    IndexConfiguration,
+    MatmulBwdConfiguration,
+    MatmulSingleConfiguration,
+)
+from oracle import kernels as oracle
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-4, 1e-5
+
+
+def assert_close(actual: torch.Tensor, expected: np.ndarray, rtol=RTOL, atol=ATOL):
+    actual = actual.detach().cpu().double().numpy()
+    assert actual.shape == expected.shape
+    err = np.abs(actual - expected)
+    tol = atol + rtol * np.abs(expected)
+    worst = np.unravel_index(np.argmax(err - tol), err.shape) if err.size else None
+    assert np.all(err <= tol), (
+        f"max violation at {worst}: got {actual[worst]}, expected {expected[worst]}, "
+        f"err {err[worst]:.3e} > tol {tol[worst]:.3e}"
+    )
+
+
+@pytest.mark.parametrize("col_blocks", [1, 2])
+def test_matmul(example_data, col_blocks):
+    d = example_data
+    args = (d.x1, d.x2, d.rhs, d.params, d.start, d.end)
+    defines = MatmulSingleConfiguration(d.kernel_type).make_config(args)
+    assert "MATMUL_COL_BLOCKS" in defines
+    defines["MATMUL_COL_BLOCKS"] = col_blocks
+    result = load_native("matmul", defines).call(*args)
+    a = d.numpy()
+    expected = oracle.matmul(d.kernel_type, a["x1"], a["x2"], a["rhs"], a["params"], a["start"], a["end"])
+    assert_close(result, expected)
+
+
+@pytest.mark.parametrize("variant,rows", [("valu", None), ("mfma", 16), ("mfma", 32), ("mfma", 64), ("mfma", 128)])
+def test_matmul_variants(example_data, variant, rows):
+    d = example_data
+    args = (d.x1, d.x2, d.rhs, d.params, d.start, d.end)
+    defines = MatmulSingleConfiguration(d.kernel_type).make_config(args)
+    defines["MATMUL_VARIANT"] = variant
+    if rows is not None:
+        defines["MATMUL_ROWS_PER_WAVE"] = rows
+    result = load_native("matmul", defines).call(*args)
+    a = d.numpy()
+    expected = oracle.matmul(d.kernel_type, a["x1"], a["x2"], a["rhs"], a["params"], a["start"], a["end"])
+    assert_close(result, expected)
+
+
+def _grad_tolerance(expected):
+    # Gradients are sums over up to m*n terms of mixed sign: compare relative to the largest
+    # component of each batch item's gradient as well as elementwise.
+    scale = np.max(np.abs(expected), axis=-1, keepdims=True)
+    return ATOL + RTOL * np.maximum(np.abs(expected), scale)
+
+
+def test_matmul_bwd(example_data):
+    d = example_data
+    out_grad = torch.randn(*d.params.shape[:-1], d.x1.shape[-1], d.rhs.shape[-1])
+    out_grad = (out_grad / torch.linalg.norm(out_grad, dim=(-2, -1), keepdim=True)).to(d.x1.device)
+    args = (d.x1, d.x2, d.rhs, d.params, d.start, d.end, out_grad)
+    defines = MatmulBwdConfiguration(d.kernel_type).make_config(args)
+    result = load_native("matmul_bwd", defines).call(*args)
+    a = d.numpy()
+    expected = oracle.param_grad(d.kernel_type, a["x1"], a["x2"], out_grad.cpu().numpy(), a["rhs"],
+                                 a["params"], a["start"], a["end"])
+    err = np.abs(result.cpu().double().numpy() - expected)
+    assert np.all(err <= _grad_tolerance(expected)), (result.cpu().numpy(), expected)
+
+
+def test_bilinear_derivative(example_data):
+    d = example_data
+    left = torch.randn(*d.x1.shape, 5)
+    left = (left / torch.linalg.norm(left, dim=-2, keepdim=True)).to(d.x1.device)
+    right = torch.randn(*d.x2.shape, 5)
+    right = (right / torch.linalg.norm(right, dim=-2, keepdim=True)).to(d.x1.device)
+    args = (d.x1, d.x2, left, right, d.params, d.start, d.end)
+    defines = BilinearDerivativeConfiguration(d.kernel_type).make_config(args)
+    result = load_native("bilinear_derivative", defines).call(*args)
+    a = d.numpy()
+    expected = oracle.param_grad(d.kernel_type, a["x1"], a["x2"], left.cpu().numpy(),
+                                 right.cpu().numpy(), a["params"], a["start"], a["end"])
+    err = np.abs(result.cpu().double().numpy() - expected)
+    assert np.all(err <= _grad_tolerance(expected)), (result.cpu().numpy(), expected)
+
+
+@pytest.mark.square
+@pytest.mark.parametrize("shape", [(100,), (5, 101)])
+def test_index(example_data, shape):
+    d = example_data
+    device = d.x1.device
+    m, n = d.x1.shape[-1], d.x2.shape[-1]
+    batch_indices = tuple(
+        torch.randint(0, size, shape, dtype=torch.int32).to(device) for size in d.params.shape[:-1]
+    )
+    row_index = torch.randint(0, m, shape, dtype=torch.int32).to(device)
+    col_index = torch.randint(0, n, shape, dtype=torch.int32).to(device)
+    args = (d.x1, d.x2, d.params, d.start, d.end, batch_indices, row_index, col_index)
+    defines = IndexConfiguration(d.kernel_type).make_config(args)
+    result = load_native("index", defines).call(*args)
+    a = d.numpy()
+    expected = oracle.index(d.kernel_type, a["x1"], a["x2"], a["params"], a["start"], a["end"],
+                            [b.cpu().numpy() for b in batch_indices], row_index.cpu().numpy(),
+                            col_index.cpu().numpy())
+    assert_close(result, expected)
+    # entries outside the pattern are exactly zero
+    assert torch.all(result[torch.from_numpy(expected == 0.0).to(device)] == 0.0)
