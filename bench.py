@@ -1,0 +1,216 @@
+#!/usr/bin/env python3
+"""Headline benchmark: sparse spectral K(x, x) @ rhs, n = 100 000, k = 16, batch 8, one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload headline|c1|c2|c5]
+                    [--variant auto|mfma|valu] [--no-cpu-baseline]
+
+A step is one call of the matmul operator over the whole batch with inputs resident in HBM.
+Prints one JSON line: kernel-pair evaluations per second (``value``), the roofline of the
+forward kernel against the MI355X fp32 peak (157.3 TFLOP/s, vector = matrix fp32), and the
+CPU baseline (dense build-K-then-matmul in fp32 torch on the host cores, bounded sample).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_FP32_TFLOPS = 157.3  # 256 CU x 256 flop/clk x 2.4 GHz; fp32 MFMA peak is the same figure
+
+WORKLOADS = {
+    # name: kernel, n, extent, batch, k, cutoff factor (x max lengthscale) or absolute, seed
+    "headline": dict(kernel="spectral", n=100_000, extent=10_000.0, batch=8, k=16, cutoff_l=6.0, seed=1000,
+                     label="spectral K@rhs n=100000 k=16 batch=8 x~U[0,10000) cutoff=6*l_max"),
+    "c1": dict(kernel="rbf", n=4096, extent=100.0, batch=0, k=1, cutoff_abs=8.0, seed=1001,
+               label="rbf K@rhs n=4096 k=1 l=sigma=1 cutoff=8"),
+    "c2": dict(kernel="spectral", n=20_000, extent=2000.0, batch=4, k=16, cutoff_l=6.0, seed=1002,
+               label="spectral K@rhs n=20000 k=16 batch=4 cutoff=6*l_max"),
+    "c5": dict(kernel="spectral", n=1_000_000, extent=100_000.0, batch=8, k=32, cutoff_l=5.0, seed=1005,
+               label="spectral K@rhs n=1000000 k=32 batch=8 cutoff=5*l_max"),
+}
+
+FLOPS_PER_PAIR = {"rbf": lambda k: 5 + 2 * k, "spectral": lambda k: 8 + 2 * k,
+                  "locally_periodic": lambda k: 10 + 2 * k}
+
+
+def make_workload(name: str, batch_override=None):
+    """Seeded CPU generation (so the GPU run and the CPU baseline see identical bits)."""
+    import torch
+
+    w = dict(WORKLOADS[name])
+    if batch_override is not None:
+        w["batch"] = batch_override
+        w["label"] += f" [batch overridden to {batch_override}]"
+    g = torch.Generator().manual_seed(w["seed"])
+    n, batch = w["n"], w["batch"]
+    x = torch.sort(torch.rand(n, generator=g) * w["extent"])[0]
+    bshape = (batch,) if batch else ()
+    u = lambda lo, hi: lo + (hi - lo) * torch.rand(bshape, generator=g)
+    if w["kernel"] == "spectral":
+        params = torch.stack([u(0.5, 2.0), u(0.05, 0.5), u(0.5, 2.0)], dim=-1)
+    else:
+        params = torch.stack([torch.ones(bshape), torch.ones(bshape)], dim=-1)
+    rhs = torch.randn(n, w["k"], generator=g)
+    cutoff = w["cutoff_abs"] if "cutoff_abs" in w else w["cutoff_l"] * float(params[..., 0].max())
+    return w, x, params.float(), rhs, cutoff
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="headline", choices=sorted(WORKLOADS))
+    ap.add_argument("--variant", default="auto", choices=["auto", "mfma_f32", "mfma_f16", "valu"])
+    ap.add_argument("--rows-per-wave", type=int, default=0)
+    ap.add_argument("--col-splits", type=int, default=0)
+    ap.add_argument("--batch", type=int, default=None, help="override the number of batch items")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU; --gpus must be 1 "
+              "(the path has no collective or multi-GPU part).", file=sys.stderr)
+        return 2
+
+    import torch
+
+    from kernel_matmul_amd import _native
+    from kernel_matmul_amd.compile import load_native
+    from kernel_matmul_amd.configurations import MatmulSingleConfiguration
+    from kernel_matmul_amd.ranges import make_ranges
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 2
+    _native.load_library()  # fail loudly if the HIP library is missing
+    device = torch.device("cuda:0")
+
+    w, x_cpu, params_cpu, rhs_cpu, cutoff = make_workload(args.workload, args.batch)
+    n, k, batch = w["n"], w["k"], w["batch"]
+    bshape = (batch,) if batch else ()
+    start_cpu, end_cpu = make_ranges(cutoff, x_cpu)  # symmetric pattern, block 128
+    row_blocks = start_cpu.shape[-1]
+    rows_in_block = torch.clamp(n - 128 * torch.arange(row_blocks), max=128)
+    pairs_per_item = int((rows_in_block * (end_cpu - start_cpu)).sum())
+    pairs = pairs_per_item * max(batch, 1)
+    flops_per_pair = FLOPS_PER_PAIR[w["kernel"]](k)
+
+    x = x_cpu.to(device)
+    rhs = rhs_cpu.to(device)
+    params = params_cpu.to(device)
+    start, end = start_cpu.to(device), end_cpu.to(device)
+    # batch items share x, rhs and the pattern (stride-0 views), as KernelMatmulLinearOperator passes them
+    xb = x.expand(*bshape, n)
+    rhsb = rhs.expand(*bshape, n, k)
+    startb = start.expand(*bshape, row_blocks)
+    endb = end.expand(*bshape, row_blocks)
+    op_args = (xb, xb, rhsb, params, startb, endb)
+
+    defines = MatmulSingleConfiguration(w["kernel"]).make_config(op_args)
+    if args.variant != "auto":
+        defines["MATMUL_VARIANT"] = args.variant
+    if args.rows_per_wave:
+        defines["MATMUL_ROWS_PER_WAVE"] = args.rows_per_wave
+    if args.col_splits:
+        defines["MATMUL_COL_BLOCKS"] = args.col_splits
+    op = load_native("matmul", defines)
+
+    for _ in range(args.warmup):
+        out = op.call(*op_args)
+    torch.cuda.synchronize()
+
+    # Whole-step wall time and, on the launch stream, per-launch event time of the kernel.
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+              for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for e0, e1 in events:
+        e0.record()
+        out = op.call(*op_args)
+        e1.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    kernel_ms = sorted(e0.elapsed_time(e1) for e0, e1 in events)
+    kernel_ms_avg = sum(kernel_ms) / len(kernel_ms)
+    kernel_ms_med = kernel_ms[len(kernel_ms) // 2]
+
+    value = pairs / (ms_per_step * 1e-3)
+    achieved_tflops = pairs * flops_per_pair / (kernel_ms_avg * 1e-3) / 1e12
+
+    traffic = None
+    traffic_path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if os.path.exists(traffic_path):
+        with open(traffic_path) as f:
+            traffic = json.load(f).get(args.workload, {}).get("bytes_per_launch")
+
+    result = {
+        "metric": "kernel-pair evaluations/s (sparse spectral K@rhs, n=100k, k=16, 1 MI355X)",
+        "value": value,
+        "unit": "pairs/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": w["label"],
+            "pairs_per_step": pairs,
+            "flops_per_pair": flops_per_pair,
+            "variant": op.defines.get("MATMUL_VARIANT", "auto (split-fp16 MFMA)"),
+            "seed": w["seed"],
+        },
+        "roofline": {
+            "bound": "mfma",
+            "kernel": {"auto": "km::fwd_mfma_f16", "mfma_f16": "km::fwd_mfma_f16", "mfma_f32": "km::fwd_mfma_f32", "valu": "km::fwd_valu"}[args.variant],
+            "achieved": achieved_tflops,
+            "peak": PEAK_FP32_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": achieved_tflops / PEAK_FP32_TFLOPS,
+            "traffic": traffic,
+            "kernel_ms_avg": kernel_ms_avg,
+            "kernel_ms_median": kernel_ms_med,
+            "pairs_per_s_kernel": pairs / (kernel_ms_avg * 1e-3),
+            "note": "fp32 vector peak == fp32 MFMA peak (157.3 TFLOP/s); evaluation runs on VALU, "
+                    "contraction on fp32 MFMA; flops = pairs * (8 + 2k), transcendental = 1",
+        },
+    }
+
+    if not args.no_cpu_baseline:
+        from oracle import dense_cpu
+
+        p0 = params_cpu[0] if batch else params_cpu
+        sec, in_band, dense_pairs, slabs, rows = dense_cpu.time_masked_matmul(
+            w["kernel"], x_cpu, x_cpu, rhs_cpu, p0, start_cpu, end_cpu, args.cpu_seconds)
+        got = (out[0] if batch else out)[: rows.shape[0]].cpu()
+        err = (got - rows).abs().max().item()
+        result["cpu_baseline"] = {
+            "value": in_band / sec,
+            "unit": "pairs/s",
+            "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"dense fp32 torch build-K-then-matmul of the first {rows.shape[0]} rows "
+                      f"({slabs} slabs of 1024 rows x {n} cols) of batch item 0; "
+                      f"{sec:.1f} s; dense pairs/s {dense_pairs / sec:.3e}; "
+                      f"max |gpu - cpu| on these rows {err:.2e}; os.cpu_count()={os.cpu_count()}",
+        }
+
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -146,7 +146,9 @@ def check_cuda_int32(x: Tensor) -> None:
 def check_float(x: Tensor) -> None:
     # The reference gets this from mutable_data_ptr<float>() (native/common/accessor.cuh:9).
     if x.dtype != torch.float32:
-        name = str(x.dtype).replace("torch.", "")
+        names = {torch.float64: "Double", torch.float16: "Half", torch.bfloat16: "BFloat16",
+                 torch.int32: "Int", torch.int64: "Long"}
+        name = names.get(x.dtype, str(x.dtype).replace("torch.", ""))
         raise RuntimeError(f"expected scalar type Float but found {name}")
 
 

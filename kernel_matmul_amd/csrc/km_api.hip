@@ -84,9 +84,9 @@ static const long long TARGET_WAVES = 4096;
 static int make_plan(const MatmulProblem& p, const km_launch_options* opt, MatmulPlan* plan) {
     int variant = opt ? opt->variant : KM_VARIANT_AUTO;
     if (variant == KM_VARIANT_AUTO) {
-        variant = KM_VARIANT_MFMA;
+        variant = KM_VARIANT_MFMA_F16;
     }
-    if (variant != KM_VARIANT_VALU && variant != KM_VARIANT_MFMA) {
+    if (variant != KM_VARIANT_VALU && variant != KM_VARIANT_MFMA_F32 && variant != KM_VARIANT_MFMA_F16) {
         return fail(KM_ERR_INVALID_ARGUMENT, "km_matmul: unknown variant %d", variant);
     }
     plan->variant = variant;

@@ -27,16 +27,22 @@ struct BatchStrides {
     long long s[KM_MAX_BATCH_RANK];
 };
 
-__device__ __forceinline__ void batch_multi_index(const BatchShape& shape, long long flat,
+__device__ __forceinline__ void batch_multi_index(const BatchShape& shape, long long flat_index,
                                                   int (&idx)[KM_MAX_BATCH_RANK]) {
+    // The number of batch items is below 2^31, so 32-bit division is enough.
+    unsigned flat = (unsigned)flat_index;
 #pragma unroll
     for (int d = KM_MAX_BATCH_RANK - 1; d >= 0; d--) {
+        idx[d] = 0;
         if (d < shape.rank) {
-            const int size = shape.sizes[d];
-            idx[d] = (int)(flat % size);
-            flat /= size;
-        } else {
-            idx[d] = 0;
+            if (d == 0) {
+                idx[0] = (int)flat;
+            } else {
+                const unsigned size = (unsigned)shape.sizes[d];
+                const unsigned q = flat / size;
+                idx[d] = (int)(flat - q * size);
+                flat = q;
+            }
         }
     }
 }

@@ -7,7 +7,7 @@
 
 namespace km {
 
-enum { KM_VARIANT_AUTO = 0, KM_VARIANT_VALU = 1, KM_VARIANT_MFMA = 2 };
+enum { KM_VARIANT_AUTO = 0, KM_VARIANT_VALU = 1, KM_VARIANT_MFMA_F32 = 2, KM_VARIANT_MFMA_F16 = 3 };
 
 struct MatmulProblem {
     int kernel_type;
@@ -32,7 +32,7 @@ struct MatmulProblem {
 
 // Which ahead-of-time instantiation runs and with what decomposition.
 struct MatmulPlan {
-    int variant;     // KM_VARIANT_VALU or KM_VARIANT_MFMA
+    int variant;     // KM_VARIANT_VALU, KM_VARIANT_MFMA_F32 or KM_VARIANT_MFMA_F16
     int k_chunk;     // rhs columns handled per workgroup (MFMA: 16/32/64, VALU: 4/8/16)
     int row_groups;  // MFMA: groups of 16 rows per wavefront (1, 2, 4, 8)
     int col_splits;  // MFMA: wavefronts per workgroup sharing one column range (1, 2, 4, 8)

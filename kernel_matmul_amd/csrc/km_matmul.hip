@@ -1,19 +1,30 @@
 // Forward operator: out = K(x1, x2) @ rhs over per-row-block column ranges, K evaluated on
-// the fly.  Two gfx950 implementations of the same contract:
+// the fly.  Three gfx950 implementations of the same contract (what
+// native/matmul/matmul.cu:13-157 of the reference computes):
 //
-//   fwd_mfma : each lane evaluates K entries directly in the A-operand layout of
-//              v_mfma_f32_16x16x4_f32 and the K-tile x rhs-tile contraction runs on the
-//              matrix pipe.  No LDS staging is needed: a wavefront owns whole rows, every
-//              x2 / rhs element of its column range is loaded exactly once per wavefront
-//              straight into the B-operand layout.
-//   fwd_valu : one row per lane, the contraction is v_fma_f32 with wave-uniform x2 / rhs
-//              operands fetched through the scalar (read-only) path.
+//   fwd_mfma_f32 : each lane evaluates K entries directly in the A-operand layout of
+//                  v_mfma_f32_16x16x4_f32; the K-tile x rhs-tile contraction is an fp32 MFMA.
+//   fwd_mfma_f16 : K entries and rhs are each split into two fp16 terms (hi + lo, 22
+//                  significant bits) and the contraction is three v_mfma_f32_16x16x32_f16
+//                  (hi*hi + hi*lo + lo*hi) accumulating in fp32.  On gfx950 the fp32 MFMA
+//                  occupies the same issue slots as the VALU that evaluates K, the fp16 MFMA
+//                  does not, so this is the faster variant.
+//   fwd_valu     : one row per lane, contraction with v_fma_f32 on wave-uniform x2 / rhs
+//                  operands fetched through the scalar (read-only) path.
 //
-// Computes what native/matmul/matmul.cu:13-157 of the reference computes.
+// None of them stages tiles in LDS: a wavefront owns whole rows, so every x2 / rhs element
+// of its column range is loaded once per wavefront, coalesced, straight into the operand
+// layout.  LDS only carries the fixed-order reduction when several wavefronts share a row
+// range.
+#include "km_batch.h"
 #include "km_common.h"
 #include "km_launch.h"
 
 namespace km {
+
+typedef _Float16 half8v __attribute__((ext_vector_type(8)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef float float2v __attribute__((ext_vector_type(2)));
 
 struct FwdArgs {
     BatchShape batch;
@@ -33,161 +44,47 @@ struct FwdArgs {
     long long x1_s, x2_s, rhs_s0, rhs_s1, params_s, start_s, end_s;
 };
 
-// ---------------------------------------------------------------------------------------
-// MFMA variant.
-//
-// v_mfma_f32_16x16x4_f32 operand layout (lane l of 64):
-//   A[i][kk] (16x4)  : i = l % 16, kk = l / 16          -> K(x1[row i], x2[col kk])
-//   B[kk][j] (4x16)  : kk = l / 16, j = l % 16          -> rhs[col kk][rhs column j]
-//   D[i][j]  (16x16) : i = 4 * (l / 16) + v, j = l % 16 -> out[row i][rhs column j], v = 0..3
-//
-// A wavefront owns R groups of 16 rows and G groups of 16 rhs columns and walks its column
-// range 4 columns per step: per step a lane loads one x2 value and G rhs values, evaluates
-// R kernel entries and issues R*G MFMAs.  With S > 1 the S wavefronts of a workgroup split
-// the column range and combine their accumulators through LDS in a fixed order.
-// ---------------------------------------------------------------------------------------
-template <int KT, int G, int R>
-__global__ void __launch_bounds__(512) fwd_mfma(const FwdArgs a) {
-    extern __shared__ float lds[];
+// Per-wavefront view of the problem, shared by the three kernels.
+struct WaveView {
+    long long b;
+    int row_block;
+    const float* x1;
+    const float* x2;
+    const float* rhs;
+    const float* params;
+    int range_start;
+    int range_end;
+};
 
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int S = blockDim.x >> 6;
-    const int li = lane & 15;
-    const int kk = lane >> 4;
-
-    const long long item = xcd_item(blockIdx.x, a.items_per_xcd);
-    if (blockIdx.x / KM_NUM_XCD >= a.items_per_xcd || item >= a.total_items) {
-        return;
-    }
-    const long long b = item % a.num_batches;
+__device__ __forceinline__ WaveView wave_view(const FwdArgs& a, long long item, int chunks_per_block,
+                                              int* chunk_in_block) {
+    WaveView w;
+    w.b = item % a.num_batches;
     const int chunk = (int)(item / a.num_batches);
-    const int row_block = chunk / a.chunks_per_block;
-    const int row0 = row_block * KM_BLOCK_SIZE + (chunk % a.chunks_per_block) * (16 * R);
-    const int kbase = blockIdx.y * (16 * G);
-
+    w.row_block = chunk / chunks_per_block;
+    *chunk_in_block = chunk % chunks_per_block;
     int bidx[KM_MAX_BATCH_RANK];
-    batch_multi_index(a.batch, b, bidx);
-    const float* __restrict__ x1 = a.x1 + batch_offset(a.batch, a.x1_bs, bidx);
-    const float* __restrict__ x2 = a.x2 + batch_offset(a.batch, a.x2_bs, bidx);
-    const float* __restrict__ rhs = a.rhs + batch_offset(a.batch, a.rhs_bs, bidx);
-    const float* __restrict__ params = a.params + batch_offset(a.batch, a.params_bs, bidx);
+    batch_multi_index(a.batch, w.b, bidx);
+    w.x1 = a.x1 + batch_offset(a.batch, a.x1_bs, bidx);
+    w.x2 = a.x2 + batch_offset(a.batch, a.x2_bs, bidx);
+    w.rhs = a.rhs + batch_offset(a.batch, a.rhs_bs, bidx);
+    w.params = a.params + batch_offset(a.batch, a.params_bs, bidx);
     // Clamped to the valid columns: a symmetric pattern over fewer points than one block
     // reports end = block size > n (native/ranges/ranges.cpp:82-93 of the reference).
-    const int range_start =
-        max(a.start[batch_offset(a.batch, a.start_bs, bidx) + row_block * a.start_s], 0);
-    const int range_end =
-        min(a.end[batch_offset(a.batch, a.end_bs, bidx) + row_block * a.end_s], a.n);
+    w.range_start = max(a.start[batch_offset(a.batch, a.start_bs, bidx) + w.row_block * a.start_s], 0);
+    w.range_end = min(a.end[batch_offset(a.batch, a.end_bs, bidx) + w.row_block * a.end_s], a.n);
+    return w;
+}
 
-    const KernelConsts kc = make_consts<KT>(params, a.params_s, true);
-
-    // This wavefront's share of the column range, in whole steps of 4 columns.
-    int col_begin = range_start;
-    int col_end = range_end;
-    if (S > 1) {
-        const int width = range_end - range_start;
-        const int per_wave = ((width + S - 1) / S + 3) & ~3;
-        col_begin = range_start + wave * per_wave;
-        col_end = min(range_end, col_begin + per_wave);
-    }
-
-    float x1v[R];
-#pragma unroll
-    for (int r = 0; r < R; r++) {
-        const int row = min(row0 + 16 * r + li, a.m - 1);
-        x1v[r] = x1[(long long)row * a.x1_s];
-    }
-
-    float4v acc[R][G];
-#pragma unroll
-    for (int r = 0; r < R; r++) {
-#pragma unroll
-        for (int g = 0; g < G; g++) {
-            acc[r][g] = (float4v){0.0f, 0.0f, 0.0f, 0.0f};
-        }
-    }
-
-    bool colmask[G];
-#pragma unroll
-    for (int g = 0; g < G; g++) {
-        colmask[g] = kbase + 16 * g + li < a.k;
-    }
-    const float* __restrict__ rhs_lane = rhs + (long long)(kbase + li) * a.rhs_s1;
-
-    // Software pipeline: operands of step t+1 are requested before step t is evaluated.
-    int col = col_begin + kk;
-    float x2v = 0.0f;
-    float bv[G];
-#pragma unroll
-    for (int g = 0; g < G; g++) {
-        bv[g] = 0.0f;
-    }
-    if (col < col_end) {
-        x2v = x2[(long long)col * a.x2_s];
-#pragma unroll
-        for (int g = 0; g < G; g++) {
-            if (colmask[g]) {
-                bv[g] = rhs_lane[(long long)col * a.rhs_s0 + (long long)(16 * g) * a.rhs_s1];
-            }
-        }
-    }
-
-    for (int c0 = col_begin; c0 < col_end; c0 += 4) {
-        const int ncol = col + 4;
-        float x2n = x2v;  // stays finite for masked-out lanes; their rhs operand is 0
-        float bn[G];
-#pragma unroll
-        for (int g = 0; g < G; g++) {
-            bn[g] = 0.0f;
-        }
-        if (ncol < col_end) {
-            x2n = x2[(long long)ncol * a.x2_s];
-#pragma unroll
-            for (int g = 0; g < G; g++) {
-                if (colmask[g]) {
-                    bn[g] = rhs_lane[(long long)ncol * a.rhs_s0 + (long long)(16 * g) * a.rhs_s1];
-                }
-            }
-        }
-
-#pragma unroll
-        for (int r = 0; r < R; r++) {
-            const float kv = kernel_value<KT>(x1v[r], x2v, kc);
-#pragma unroll
-            for (int g = 0; g < G; g++) {
-                acc[r][g] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv, bv[g], acc[r][g], 0, 0, 0);
-            }
-        }
-
-        col = ncol;
-        x2v = x2n;
-#pragma unroll
-        for (int g = 0; g < G; g++) {
-            bv[g] = bn[g];
-        }
-    }
-
-    float* __restrict__ out = a.out + b * (long long)a.m * a.k;
-
-    if (S == 1) {
-#pragma unroll
-        for (int r = 0; r < R; r++) {
-#pragma unroll
-            for (int g = 0; g < G; g++) {
-#pragma unroll
-                for (int v = 0; v < 4; v++) {
-                    const int row = row0 + 16 * r + 4 * kk + v;
-                    if (row < a.m && colmask[g]) {
-                        out[(long long)row * a.k + kbase + 16 * g + li] = acc[r][g][v] * kc.sgn;
-                    }
-                }
-            }
-        }
-        return;
-    }
-
-    // Cross-wavefront reduction: lds[wave][slot][lane], slot = (r * G + g) * 4 + v.
+// Fixed-order reduction of the S wavefronts' accumulators through LDS and the masked store.
+// lds[wave][slot][lane], slot = (r * G + g) * 4 + v in the MFMA D layout.
+template <int G, int R>
+__device__ __forceinline__ void reduce_and_store(const float4v (&acc)[R][G], float* lds, int S,
+                                                 int wave, int lane, float* __restrict__ out,
+                                                 int row0, int kbase, int m, int k) {
     constexpr int SLOTS = R * G * 4;
+    const int li = lane & 15;
+    const int kk = lane >> 4;
     float* mine = lds + (size_t)wave * SLOTS * 64;
 #pragma unroll
     for (int r = 0; r < R; r++) {
@@ -210,9 +107,395 @@ __global__ void __launch_bounds__(512) fwd_mfma(const FwdArgs a) {
         const int r = (slot >> 2) / G;
         const int row = row0 + 16 * r + 4 * kk + v;
         const int c = kbase + 16 * g + li;
-        if (row < a.m && c < a.k) {
-            out[(long long)row * a.k + c] = sum * kc.sgn;
+        if (row < m && c < k) {
+            out[(long long)row * k + c] = sum;
         }
+    }
+}
+
+template <int G, int R>
+__device__ __forceinline__ void store_direct(const float4v (&acc)[R][G], int lane,
+                                             float* __restrict__ out, int row0, int kbase, int m,
+                                             int k) {
+    const int li = lane & 15;
+    const int kk = lane >> 4;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            const int c = kbase + 16 * g + li;
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const int row = row0 + 16 * r + 4 * kk + v;
+                if (row < m && c < k) {
+                    out[(long long)row * k + c] = acc[r][g][v];
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// fp32 MFMA variant.
+//
+// v_mfma_f32_16x16x4_f32 operand layout (lane l of 64):
+//   A[i][kk] (16x4)  : i = l % 16, kk = l / 16          -> K(x1[row i], x2[col kk])
+//   B[kk][j] (4x16)  : kk = l / 16, j = l % 16          -> rhs[col kk][rhs column j]
+//   D[i][j]  (16x16) : i = 4 * (l / 16) + v, j = l % 16 -> out[row i][rhs column j], v = 0..3
+//
+// A wavefront owns R groups of 16 rows and G groups of 16 rhs columns and walks its column
+// range 4 columns per step: per step a lane loads one x2 value and G rhs values, evaluates
+// R kernel entries and issues R*G MFMAs.  With S > 1 the S wavefronts of a workgroup split
+// the column range.
+// ---------------------------------------------------------------------------------------
+template <int KT, int G, int R>
+__global__ void __launch_bounds__(512) fwd_mfma_f32(const FwdArgs a) {
+    extern __shared__ float lds[];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int S = blockDim.x >> 6;
+    const int li = lane & 15;
+    const int kk = lane >> 4;
+
+    const long long item = xcd_item(blockIdx.x, a.items_per_xcd);
+    if (item >= a.total_items) {
+        return;
+    }
+    int chunk_in_block;
+    const WaveView w = wave_view(a, item, a.chunks_per_block, &chunk_in_block);
+    const int row0 = w.row_block * KM_BLOCK_SIZE + chunk_in_block * (16 * R);
+    const int kbase = blockIdx.y * (16 * G);
+
+    const KernelConsts kc = make_consts<KT>(w.params, a.params_s, true);
+
+    // This wavefront's share of the column range, in whole steps of 4 columns.
+    int col_begin = w.range_start;
+    int col_end = w.range_end;
+    if (S > 1) {
+        const int width = max(w.range_end - w.range_start, 0);
+        const int per_wave = ((width + S - 1) / S + 3) & ~3;
+        col_begin = w.range_start + wave * per_wave;
+        col_end = min(w.range_end, col_begin + per_wave);
+    }
+
+    float x1v[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int row = min(row0 + 16 * r + li, a.m - 1);
+        x1v[r] = w.x1[(long long)row * a.x1_s];
+    }
+
+    float4v acc[R][G];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            acc[r][g] = (float4v){0.0f, 0.0f, 0.0f, 0.0f};
+        }
+    }
+
+    bool colmask[G];
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        colmask[g] = kbase + 16 * g + li < a.k;
+    }
+
+    // Operand pointers advance by 4 columns per step.
+    const float* x2p = w.x2 + (long long)(col_begin + kk) * a.x2_s;
+    const float* rp = w.rhs + (long long)(col_begin + kk) * a.rhs_s0 + (long long)(kbase + li) * a.rhs_s1;
+    const long long x2_step = 4 * a.x2_s;
+    const long long r_step = 4 * a.rhs_s0;
+    const long long g_step = 16 * a.rhs_s1;
+
+    // Software pipeline: operands of step t+1 are requested before step t is evaluated.
+    int col = col_begin + kk;
+    float x2v = 0.0f;
+    float bv[G];
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        bv[g] = 0.0f;
+    }
+    if (col < col_end) {
+        x2v = *x2p;
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            if (colmask[g]) {
+                bv[g] = rp[g * g_step];
+            }
+        }
+    }
+
+    for (int c0 = col_begin; c0 < col_end; c0 += 4) {
+        col += 4;
+        x2p += x2_step;
+        rp += r_step;
+        float x2n = x2v;  // stays finite for masked-out lanes; their rhs operand is 0
+        float bn[G];
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            bn[g] = 0.0f;
+        }
+        if (col < col_end) {
+            x2n = *x2p;
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                if (colmask[g]) {
+                    bn[g] = rp[g * g_step];
+                }
+            }
+        }
+
+        float kv[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            kv[r] = kernel_value<KT>(x1v[r], x2v, kc);
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                acc[r][g] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv[r], bv[g], acc[r][g], 0, 0, 0);
+            }
+        }
+
+        x2v = x2n;
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            bv[g] = bn[g];
+        }
+    }
+
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            acc[r][g] *= kc.sgn;
+        }
+    }
+    float* __restrict__ out = a.out + w.b * (long long)a.m * a.k;
+    if (S == 1) {
+        store_direct<G, R>(acc, lane, out, row0, kbase, a.m, a.k);
+    } else {
+        reduce_and_store<G, R>(acc, lds, S, wave, lane, out, row0, kbase, a.m, a.k);
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// Split-fp16 MFMA variant.
+//
+// v_mfma_f32_16x16x32_f16 operand layout (lane l of 64, 8 halves per operand register set):
+//   A[i][8 kk + t] (16x32) : i = l % 16, kk = l / 16, t = 0..7 -> K(x1[row i], x2[col 8 kk + t])
+//   B[8 kk + t][j] (32x16) : j = l % 16                         -> rhs[col 8 kk + t][rhs column j]
+//   D as for the fp32 instruction.
+//
+// Every fp32 factor v is written as hi + lo with hi = fp16(v) and lo = fp16(v - hi)
+// (round-to-nearest-even, v_cvt_pk_f16_f32), i.e. 22 significant bits, and the product is
+// taken as hi*hi + hi*lo + lo*hi in the fp32 accumulator; the dropped lo*lo term is below
+// 2^-22 relative.  To keep both factors inside the fp16 exponent range
+//   - K is evaluated without sigma and scaled by 2^14 (folded into the exponent of the
+//     base-2 exponential, so it costs nothing): |K| <= 2^14;
+//   - each rhs column is scaled by a power of two chosen per wavefront from the largest
+//     magnitude in the wavefront's column window (one pre-scan of the window).
+// Both scales and sigma are undone on the accumulators before they leave the wavefront.
+// ---------------------------------------------------------------------------------------
+#define KM_F16_KSCALE_LOG2 14
+
+template <int KT>
+__device__ __forceinline__ void kernel_pair_f16(float x1, float x2a, float x2b, const KernelConsts& c,
+                                                half2v* hi, half2v* lo) {
+    // Two neighbouring columns at once so that the conversions pack.
+    float2v kv, res;
+    float ea[2], ca[2];
+    const float x2s[2] = {x2a, x2b};
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        const float d = x1 - x2s[t];
+        const float u = d * c.s;
+        const float arg = __builtin_fmaf(-u, u, (float)KM_F16_KSCALE_LOG2);
+        if (KT == KM_KERNEL_RBF) {
+            ea[t] = __builtin_amdgcn_exp2f(arg);
+            ca[t] = 1.0f;
+        } else if (KT == KM_KERNEL_SPECTRAL) {
+            ea[t] = __builtin_amdgcn_exp2f(arg);
+            ca[t] = __builtin_amdgcn_cosf(d * c.f);
+        } else {
+            const float sn = __builtin_amdgcn_sinf(d * c.f);
+            const float wv = sn * c.cl;
+            ea[t] = __builtin_amdgcn_exp2f(__builtin_fmaf(-wv, sn, arg));
+            ca[t] = 1.0f;
+        }
+        kv[t] = KT == KM_KERNEL_SPECTRAL ? ea[t] * ca[t] : ea[t];
+    }
+    const half2v h = __builtin_convertvector(kv, half2v);
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        // Residual of the exact product where there is one (contracts to one fused op).
+        res[t] = KT == KM_KERNEL_SPECTRAL ? __builtin_fmaf(ea[t], ca[t], -(float)h[t])
+                                          : ea[t] - (float)h[t];
+    }
+    *hi = h;
+    *lo = __builtin_convertvector(res, half2v);
+}
+
+__device__ __forceinline__ void split_f16x8(const float (&v)[8], half8v* hi, half8v* lo) {
+#pragma unroll
+    for (int t = 0; t < 8; t += 2) {
+        const float2v p = {v[t], v[t + 1]};
+        const half2v h = __builtin_convertvector(p, half2v);
+        const float2v r = {v[t] - (float)h[0], v[t + 1] - (float)h[1]};
+        const half2v l = __builtin_convertvector(r, half2v);
+        (*hi)[t] = h[0];
+        (*hi)[t + 1] = h[1];
+        (*lo)[t] = l[0];
+        (*lo)[t + 1] = l[1];
+    }
+}
+
+template <int KT, int G, int R>
+__global__ void __launch_bounds__(512) fwd_mfma_f16(const FwdArgs a) {
+    extern __shared__ float lds[];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int S = blockDim.x >> 6;
+    const int li = lane & 15;
+    const int kk = lane >> 4;
+
+    const long long item = xcd_item(blockIdx.x, a.items_per_xcd);
+    if (item >= a.total_items) {
+        return;
+    }
+    int chunk_in_block;
+    const WaveView w = wave_view(a, item, a.chunks_per_block, &chunk_in_block);
+    const int row0 = w.row_block * KM_BLOCK_SIZE + chunk_in_block * (16 * R);
+    const int kbase = blockIdx.y * (16 * G);
+
+    const KernelConsts kc = make_consts<KT>(w.params, a.params_s, false);
+    const float sigma = w.params[KernelTraits<KT>::SIGMA * a.params_s];
+
+    // This wavefront's share of the column range, in whole steps of 32 columns.
+    int col_begin = w.range_start;
+    int col_end = w.range_end;
+    if (S > 1) {
+        const int width = max(w.range_end - w.range_start, 0);
+        const int per_wave = ((width + S - 1) / S + 31) & ~31;
+        col_begin = w.range_start + wave * per_wave;
+        col_end = min(w.range_end, col_begin + per_wave);
+    }
+
+    float x1v[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int row = min(row0 + 16 * r + li, a.m - 1);
+        x1v[r] = w.x1[(long long)row * a.x1_s];
+    }
+
+    bool colmask[G];
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        colmask[g] = kbase + 16 * g + li < a.k;
+    }
+    const float* __restrict__ rhs_lane = w.rhs + (long long)(kbase + li) * a.rhs_s1;
+    const long long g_step = 16 * a.rhs_s1;
+
+    // Pre-scan: largest |rhs| per rhs column over this wavefront's window -> power-of-two scale
+    // that brings the column below 2^14.
+    float scale[G], unscale[G];
+    {
+        float cmax[G];
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            cmax[g] = 0.0f;
+        }
+        for (int col = col_begin + kk; col < col_end; col += 4) {
+            const float* p = rhs_lane + (long long)col * a.rhs_s0;
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                if (colmask[g]) {
+                    cmax[g] = fmaxf(cmax[g], fabsf(p[g * g_step]));
+                }
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            cmax[g] = fmaxf(cmax[g], __shfl_xor(cmax[g], 16, 64));
+            cmax[g] = fmaxf(cmax[g], __shfl_xor(cmax[g], 32, 64));
+            // cmax < 2^e  =>  cmax * 2^(14 - e) < 2^14; the shift is clamped so that the scale
+            // and its inverse stay normal numbers.
+            const int e = cmax[g] > 0.0f ? __builtin_amdgcn_frexp_expf(cmax[g]) : KM_F16_KSCALE_LOG2;
+            const int shift = min(max(KM_F16_KSCALE_LOG2 - e, -100), 100);
+            scale[g] = __builtin_ldexpf(1.0f, shift);
+            unscale[g] = __builtin_ldexpf(sigma, -shift - KM_F16_KSCALE_LOG2);
+        }
+    }
+
+    float4v acc[R][G];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            acc[r][g] = (float4v){0.0f, 0.0f, 0.0f, 0.0f};
+        }
+    }
+
+    const int last_col = a.n - 1;
+    for (int c0 = col_begin; c0 < col_end; c0 += 32) {
+        // This lane's 8 columns of the step.  Columns past the range keep a valid x2 (clamped
+        // index) and get a zero rhs operand.
+        const int cbase = c0 + 8 * kk;
+        float x2v[8];
+        half8v bhi[G], blo[G];
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+            x2v[t] = w.x2[(long long)min(cbase + t, last_col) * a.x2_s];
+        }
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            float rv[8];
+#pragma unroll
+            for (int t = 0; t < 8; t++) {
+                const int col = cbase + t;
+                rv[t] = (col < col_end && colmask[g])
+                            ? rhs_lane[(long long)col * a.rhs_s0 + g * g_step] * scale[g]
+                            : 0.0f;
+            }
+            split_f16x8(rv, &bhi[g], &blo[g]);
+        }
+
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            half8v ahi, alo;
+#pragma unroll
+            for (int t = 0; t < 8; t += 2) {
+                half2v h, l;
+                kernel_pair_f16<KT>(x1v[r], x2v[t], x2v[t + 1], kc, &h, &l);
+                ahi[t] = h[0];
+                ahi[t + 1] = h[1];
+                alo[t] = l[0];
+                alo[t + 1] = l[1];
+            }
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                acc[r][g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahi, bhi[g], acc[r][g], 0, 0, 0);
+                acc[r][g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahi, blo[g], acc[r][g], 0, 0, 0);
+                acc[r][g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(alo, bhi[g], acc[r][g], 0, 0, 0);
+            }
+        }
+    }
+
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            acc[r][g] *= unscale[g];
+        }
+    }
+    float* __restrict__ out = a.out + w.b * (long long)a.m * a.k;
+    if (S == 1) {
+        store_direct<G, R>(acc, lane, out, row0, kbase, a.m, a.k);
+    } else {
+        reduce_and_store<G, R>(acc, lds, S, wave, lane, out, row0, kbase, a.m, a.k);
     }
 }
 
@@ -224,29 +507,16 @@ __global__ void __launch_bounds__(512) fwd_mfma(const FwdArgs a) {
 template <int KT, int KC>
 __global__ void __launch_bounds__(128) fwd_valu(const FwdArgs a) {
     const long long item = xcd_item(blockIdx.x, a.items_per_xcd);
-    if (blockIdx.x / KM_NUM_XCD >= a.items_per_xcd || item >= a.total_items) {
+    if (item >= a.total_items) {
         return;
     }
-    const long long b = item % a.num_batches;
-    const int row_block = (int)(item / a.num_batches);
-    const int row = row_block * KM_BLOCK_SIZE + threadIdx.x;
+    int unused;
+    const WaveView w = wave_view(a, item, 1, &unused);
+    const int row = w.row_block * KM_BLOCK_SIZE + threadIdx.x;
     const int kbase = blockIdx.y * KC;
 
-    int bidx[KM_MAX_BATCH_RANK];
-    batch_multi_index(a.batch, b, bidx);
-    const float* __restrict__ x1 = a.x1 + batch_offset(a.batch, a.x1_bs, bidx);
-    const float* __restrict__ x2 = a.x2 + batch_offset(a.batch, a.x2_bs, bidx);
-    const float* __restrict__ rhs = a.rhs + batch_offset(a.batch, a.rhs_bs, bidx);
-    const float* __restrict__ params = a.params + batch_offset(a.batch, a.params_bs, bidx);
-    // Clamped to the valid columns: a symmetric pattern over fewer points than one block
-    // reports end = block size > n (native/ranges/ranges.cpp:82-93 of the reference).
-    const int range_start =
-        max(a.start[batch_offset(a.batch, a.start_bs, bidx) + row_block * a.start_s], 0);
-    const int range_end =
-        min(a.end[batch_offset(a.batch, a.end_bs, bidx) + row_block * a.end_s], a.n);
-
-    const KernelConsts kc = make_consts<KT>(params, a.params_s, true);
-    const float x1v = x1[(long long)min(row, a.m - 1) * a.x1_s];
+    const KernelConsts kc = make_consts<KT>(w.params, a.params_s, true);
+    const float x1v = w.x1[(long long)min(row, a.m - 1) * a.x1_s];
 
     float acc[KC];
 #pragma unroll
@@ -255,9 +525,10 @@ __global__ void __launch_bounds__(128) fwd_valu(const FwdArgs a) {
     }
 
     const int kc_valid = min(KC, a.k - kbase);
-    const float* __restrict__ rhs_base = rhs + (long long)kbase * a.rhs_s1;
+    const float* __restrict__ x2 = w.x2;
+    const float* __restrict__ rhs_base = w.rhs + (long long)kbase * a.rhs_s1;
     if (kc_valid == KC) {
-        for (int j = range_start; j < range_end; j++) {
+        for (int j = w.range_start; j < w.range_end; j++) {
             const float kv = kernel_value<KT>(x1v, x2[(long long)j * a.x2_s], kc);
             const float* __restrict__ rj = rhs_base + (long long)j * a.rhs_s0;
 #pragma unroll
@@ -266,7 +537,7 @@ __global__ void __launch_bounds__(128) fwd_valu(const FwdArgs a) {
             }
         }
     } else {
-        for (int j = range_start; j < range_end; j++) {
+        for (int j = w.range_start; j < w.range_end; j++) {
             const float kv = kernel_value<KT>(x1v, x2[(long long)j * a.x2_s], kc);
             const float* __restrict__ rj = rhs_base + (long long)j * a.rhs_s0;
 #pragma unroll
@@ -278,7 +549,7 @@ __global__ void __launch_bounds__(128) fwd_valu(const FwdArgs a) {
     }
 
     if (row < a.m) {
-        float* __restrict__ out = a.out + (b * a.m + row) * (long long)a.k + kbase;
+        float* __restrict__ out = a.out + (w.b * a.m + row) * (long long)a.k + kbase;
 #pragma unroll
         for (int c = 0; c < KC; c++) {
             if (c < kc_valid) {
@@ -292,32 +563,35 @@ __global__ void __launch_bounds__(128) fwd_valu(const FwdArgs a) {
 // Host dispatch.
 // ---------------------------------------------------------------------------------------
 template <int KT, int G, int R>
-static hipError_t launch_mfma(const FwdArgs& a, int S, unsigned grid_x, unsigned grid_y,
+static hipError_t launch_mfma(const FwdArgs& a, int variant, int S, unsigned gx, unsigned gy,
                               hipStream_t stream) {
     const size_t lds = S > 1 ? (size_t)S * R * G * 4 * 64 * sizeof(float) : 0;
-    hipLaunchKernelGGL((fwd_mfma<KT, G, R>), dim3(grid_x, grid_y, 1), dim3(64 * S, 1, 1), lds,
-                       stream, a);
+    if (variant == KM_VARIANT_MFMA_F16) {
+        hipLaunchKernelGGL((fwd_mfma_f16<KT, G, R>), dim3(gx, gy, 1), dim3(64 * S, 1, 1), lds, stream, a);
+    } else {
+        hipLaunchKernelGGL((fwd_mfma_f32<KT, G, R>), dim3(gx, gy, 1), dim3(64 * S, 1, 1), lds, stream, a);
+    }
     return hipGetLastError();
 }
 
 template <int KT, int G>
-static hipError_t launch_mfma_r(const FwdArgs& a, int R, int S, unsigned gx, unsigned gy,
-                                hipStream_t stream) {
+static hipError_t launch_mfma_r(const FwdArgs& a, int variant, int R, int S, unsigned gx,
+                                unsigned gy, hipStream_t stream) {
     switch (R) {
-        case 8: return launch_mfma<KT, G, 8>(a, S, gx, gy, stream);
-        case 4: return launch_mfma<KT, G, 4>(a, S, gx, gy, stream);
-        case 2: return launch_mfma<KT, G, 2>(a, S, gx, gy, stream);
-        default: return launch_mfma<KT, G, 1>(a, S, gx, gy, stream);
+        case 8: return launch_mfma<KT, G, 8>(a, variant, S, gx, gy, stream);
+        case 4: return launch_mfma<KT, G, 4>(a, variant, S, gx, gy, stream);
+        case 2: return launch_mfma<KT, G, 2>(a, variant, S, gx, gy, stream);
+        default: return launch_mfma<KT, G, 1>(a, variant, S, gx, gy, stream);
     }
 }
 
 template <int KT>
-static hipError_t launch_mfma_g(const FwdArgs& a, int G, int R, int S, unsigned gx, unsigned gy,
-                                hipStream_t stream) {
+static hipError_t launch_mfma_g(const FwdArgs& a, int variant, int G, int R, int S, unsigned gx,
+                                unsigned gy, hipStream_t stream) {
     switch (G) {
-        case 4: return launch_mfma_r<KT, 4>(a, R, S, gx, gy, stream);
-        case 2: return launch_mfma_r<KT, 2>(a, R, S, gx, gy, stream);
-        default: return launch_mfma_r<KT, 1>(a, R, S, gx, gy, stream);
+        case 4: return launch_mfma_r<KT, 4>(a, variant, R, S, gx, gy, stream);
+        case 2: return launch_mfma_r<KT, 2>(a, variant, R, S, gx, gy, stream);
+        default: return launch_mfma_r<KT, 1>(a, variant, R, S, gx, gy, stream);
     }
 }
 
@@ -334,18 +608,13 @@ static hipError_t launch_valu(const FwdArgs& a, int KC, unsigned gx, unsigned gy
     return hipGetLastError();
 }
 
-static void fill_strides(BatchStrides& dst, const int64_t* strides, int rank) {
-    for (int d = 0; d < KM_MAX_BATCH_RANK; d++) {
-        dst.s[d] = d < rank ? strides[d] : 0;
-    }
-}
-
 hipError_t launch_matmul(const MatmulProblem& p, const MatmulPlan& plan, hipStream_t stream) {
     FwdArgs a;
-    a.batch.rank = p.batch_rank;
-    for (int d = 0; d < KM_MAX_BATCH_RANK; d++) {
-        a.batch.sizes[d] = d < p.batch_rank ? (int)p.batch_sizes[d] : 1;
-    }
+    const int r = p.batch_rank;
+    const int64_t* const strides[6] = {p.x1_strides, p.x2_strides, p.rhs_strides,
+                                       p.params_strides, p.start_strides, p.end_strides};
+    BatchStrides* outs[6] = {&a.x1_bs, &a.x2_bs, &a.rhs_bs, &a.params_bs, &a.start_bs, &a.end_bs};
+    collapse_batch<6>(r, p.batch_sizes, strides, &a.batch, outs);
     a.num_batches = p.num_batches;
     a.m = (int)p.m;
     a.n = (int)p.n;
@@ -357,13 +626,6 @@ hipError_t launch_matmul(const MatmulProblem& p, const MatmulPlan& plan, hipStre
     a.start = p.start;
     a.end = p.end;
     a.out = p.out;
-    const int r = p.batch_rank;
-    fill_strides(a.x1_bs, p.x1_strides, r);
-    fill_strides(a.x2_bs, p.x2_strides, r);
-    fill_strides(a.rhs_bs, p.rhs_strides, r);
-    fill_strides(a.params_bs, p.params_strides, r);
-    fill_strides(a.start_bs, p.start_strides, r);
-    fill_strides(a.end_bs, p.end_strides, r);
     a.x1_s = p.x1_strides[r];
     a.x2_s = p.x2_strides[r];
     a.rhs_s0 = p.rhs_strides[r];
@@ -382,9 +644,9 @@ hipError_t launch_matmul(const MatmulProblem& p, const MatmulPlan& plan, hipStre
     }
     a.items_per_xcd = (a.total_items + KM_NUM_XCD - 1) / KM_NUM_XCD;
     const unsigned grid_x = (unsigned)(a.items_per_xcd * KM_NUM_XCD);
+    const unsigned grid_y = (unsigned)((p.k + plan.k_chunk - 1) / plan.k_chunk);
 
     if (plan.variant == KM_VARIANT_VALU) {
-        const unsigned grid_y = (unsigned)((p.k + plan.k_chunk - 1) / plan.k_chunk);
         switch (p.kernel_type) {
             case KM_KERNEL_RBF: return launch_valu<KM_KERNEL_RBF>(a, plan.k_chunk, grid_x, grid_y, stream);
             case KM_KERNEL_SPECTRAL: return launch_valu<KM_KERNEL_SPECTRAL>(a, plan.k_chunk, grid_x, grid_y, stream);
@@ -392,14 +654,13 @@ hipError_t launch_matmul(const MatmulProblem& p, const MatmulPlan& plan, hipStre
         }
     }
     const int G = plan.k_chunk / 16;
-    const unsigned grid_y = (unsigned)((p.k + plan.k_chunk - 1) / plan.k_chunk);
     switch (p.kernel_type) {
         case KM_KERNEL_RBF:
-            return launch_mfma_g<KM_KERNEL_RBF>(a, G, plan.row_groups, plan.col_splits, grid_x, grid_y, stream);
+            return launch_mfma_g<KM_KERNEL_RBF>(a, plan.variant, G, plan.row_groups, plan.col_splits, grid_x, grid_y, stream);
         case KM_KERNEL_SPECTRAL:
-            return launch_mfma_g<KM_KERNEL_SPECTRAL>(a, G, plan.row_groups, plan.col_splits, grid_x, grid_y, stream);
+            return launch_mfma_g<KM_KERNEL_SPECTRAL>(a, plan.variant, G, plan.row_groups, plan.col_splits, grid_x, grid_y, stream);
         default:
-            return launch_mfma_g<KM_KERNEL_LOCALLY_PERIODIC>(a, G, plan.row_groups, plan.col_splits, grid_x, grid_y, stream);
+            return launch_mfma_g<KM_KERNEL_LOCALLY_PERIODIC>(a, plan.variant, G, plan.row_groups, plan.col_splits, grid_x, grid_y, stream);
     }
 }
 

@@ -12,6 +12,7 @@
 // Pass 2 (param_grad_reduce): one workgroup per batch item adds the partial rows in a
 // fixed order in fp64 and applies the chain rule back to the user parameters
 // (native/common/kernel_function.cuh:221-251).  No atomics: results are reproducible.
+#include "km_batch.h"
 #include "km_common.h"
 #include "km_launch.h"
 
@@ -298,12 +299,6 @@ long long param_grad_partials_per_batch(int64_t m, long long num_batches) {
     return row_blocks * grad_col_splits(m, num_batches);
 }
 
-static void fill_strides(BatchStrides& dst, const int64_t* strides, int rank) {
-    for (int d = 0; d < KM_MAX_BATCH_RANK; d++) {
-        dst.s[d] = d < rank ? strides[d] : 0;
-    }
-}
-
 template <int KT>
 static hipError_t launch_partial(const GradArgs& a, unsigned grid_x, hipStream_t stream) {
     if (a.c <= 4) {
@@ -321,10 +316,11 @@ static hipError_t launch_partial(const GradArgs& a, unsigned grid_x, hipStream_t
 hipError_t launch_param_grad(const ParamGradProblem& p, hipStream_t stream) {
     GradArgs a;
     const int r = p.batch_rank;
-    a.batch.rank = r;
-    for (int d = 0; d < KM_MAX_BATCH_RANK; d++) {
-        a.batch.sizes[d] = d < r ? (int)p.batch_sizes[d] : 1;
-    }
+    const int64_t* const strides[7] = {p.x1_strides, p.x2_strides, p.left_strides, p.right_strides,
+                                       p.params_strides, p.start_strides, p.end_strides};
+    BatchStrides* outs[7] = {&a.x1_bs, &a.x2_bs, &a.left_bs, &a.right_bs,
+                             &a.params_bs, &a.start_bs, &a.end_bs};
+    collapse_batch<7>(r, p.batch_sizes, strides, &a.batch, outs);
     a.num_batches = p.num_batches;
     a.m = (int)p.m;
     a.n = (int)p.n;
@@ -341,13 +337,6 @@ hipError_t launch_param_grad(const ParamGradProblem& p, hipStream_t stream) {
     a.start = p.start;
     a.end = p.end;
     a.partials = (float*)p.workspace;
-    fill_strides(a.x1_bs, p.x1_strides, r);
-    fill_strides(a.x2_bs, p.x2_strides, r);
-    fill_strides(a.left_bs, p.left_strides, r);
-    fill_strides(a.right_bs, p.right_strides, r);
-    fill_strides(a.params_bs, p.params_strides, r);
-    fill_strides(a.start_bs, p.start_strides, r);
-    fill_strides(a.end_bs, p.end_strides, r);
     a.x1_s = p.x1_strides[r];
     a.x2_s = p.x2_strides[r];
     a.left_s0 = p.left_strides[r];

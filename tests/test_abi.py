@@ -1,0 +1,82 @@
+"""The C-ABI library loads, exports every function include/kernel_matmul_amd.h declares, and
+its argument validation works without touching a GPU (no compute calls here)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from kernel_matmul_amd import _native
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "kernel_matmul_amd.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(km_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    names = declared_functions()
+    for required in ("km_matmul", "km_param_grad", "km_param_grad_workspace_size", "km_index",
+                     "km_make_ranges", "km_make_ranges_symmetric", "km_transpose_ranges",
+                     "km_make_ranges_device", "km_make_ranges_symmetric_device", "km_last_error",
+                     "km_version", "km_num_params"):
+        assert required in names
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _native.load_library()
+    for name in declared_functions():
+        assert hasattr(lib, name), f"{name} declared in the header but not exported"
+
+
+def test_version_and_num_params():
+    lib = _native.load_library()
+    assert lib.km_version() >= 100
+    assert [lib.km_num_params(i) for i in range(4)] == [2, 3, 4, -1]
+
+
+def test_host_argument_validation():
+    lib = _native.load_library()
+    x = np.zeros(4, dtype=np.float32)
+    out = np.zeros(4, dtype=np.int32)
+    p = lambda a: a.ctypes.data_as(ctypes.c_void_p)
+    status = lib.km_make_ranges_symmetric(p(x), 1, 4, 1.0, 0, p(out), p(out))
+    assert status == -1 and b"block_size" in lib.km_last_error()
+    status = lib.km_make_ranges(None, None, 1, 4, 4, 1.0, 2, 0, p(out), p(out))
+    assert status == -1 and b"NULL" in lib.km_last_error()
+    status = lib.km_transpose_ranges(p(out), p(out), 1, 3, 4, 4, 2, p(out), p(out))
+    assert status == -1 and b"rows" in lib.km_last_error()
+
+
+def test_device_entry_points_reject_bad_arguments_before_launching():
+    lib = _native.load_library()
+    sizes = (ctypes.c_int64 * 1)(2)
+    # unknown kernel type
+    status = lib.km_matmul(9, 1, sizes, 4, 4, 1, None, None, None, None, None, None, None, None,
+                           None, None, None, None, None, None, None)
+    assert status == -2 and b"kernel type" in lib.km_last_error()
+    # too many batch dimensions
+    status = lib.km_matmul(0, 7, sizes, 4, 4, 1, None, None, None, None, None, None, None, None,
+                           None, None, None, None, None, None, None)
+    assert status == -2 and b"batch rank" in lib.km_last_error()
+    # NULL data pointer
+    status = lib.km_matmul(0, 1, sizes, 4, 4, 1, None, None, None, None, None, None, None, None,
+                           None, None, None, None, None, None, None)
+    assert status == -1 and b"NULL" in lib.km_last_error()
+    # empty problems are accepted and do nothing
+    assert lib.km_matmul(0, 1, sizes, 0, 4, 1, None, None, None, None, None, None, None, None,
+                         None, None, None, None, None, None, None) == 0
+    assert lib.km_param_grad_workspace_size(1, 1, sizes, 1000, 1000, 4) > 0
+    assert lib.km_param_grad_workspace_size(1, 1, sizes, 0, 1000, 4) == 0
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(_native, "_lib", None)
+    monkeypatch.setattr(_native, "LIB_PATH", "/nonexistent/libkernel_matmul_amd.so")
+    with pytest.raises(RuntimeError, match="native library not found"):
+        _native.load_library()
