@@ -259,6 +259,11 @@ def index(kernel_type: str, x1: Tensor, x2: Tensor, params: Tensor, start: Tenso
         )
     for t in (*batch_indices, row_index, col_index):
         check_cuda_int32(t)
+    if row_index.dim() == 0:  # scalar indices: treat as one entry
+        result = index(kernel_type, x1, x2, params, start, end,
+                       [b.reshape(1) for b in batch_indices], row_index.reshape(1),
+                       col_index.reshape(1))
+        return result.reshape(())
     shape = tuple(row_index.shape)
     if len(shape) < 1 or len(shape) > MAX_BATCH_RANK + 1:
         raise RuntimeError(f"index tensors must have between 1 and {MAX_BATCH_RANK + 1} dimensions")

@@ -295,8 +295,9 @@ __global__ void __launch_bounds__(512) fwd_mfma_f32(const FwdArgs a) {
 // 2^-22 relative.  To keep both factors inside the fp16 exponent range
 //   - K is evaluated without sigma and scaled by 2^14 (folded into the exponent of the
 //     base-2 exponential, so it costs nothing): |K| <= 2^14;
-//   - each rhs column is scaled by a power of two chosen per wavefront from the largest
-//     magnitude in the wavefront's column window (one pre-scan of the window).
+//   - each rhs column carries a running power-of-two scale per wavefront: when a step brings
+//     a value that would exceed 2^15 after scaling, the scale is lowered and the column's
+//     accumulators are multiplied by the (exact) ratio, so no pass over rhs is needed.
 // Both scales and sigma are undone on the accumulators before they leave the wavefront.
 // ---------------------------------------------------------------------------------------
 #define KM_F16_KSCALE_LOG2 14
@@ -352,6 +353,70 @@ __device__ __forceinline__ void split_f16x8(const float (&v)[8], half8v* hi, hal
     }
 }
 
+// One step of 32 columns: convert this lane's 8 rhs values per column group to hi/lo halves
+// (rescaling the accumulators first if a value would leave the fp16 range), then for every
+// row group evaluate 8 kernel entries, split them and issue the three MFMAs.
+template <int KT, int G, int R>
+__device__ __forceinline__ void f16_step(const float (&x2v)[8], const float (&raw)[G][8],
+                                         const float (&keep)[8], const float (&x1v)[R],
+                                         const KernelConsts& kc, const bool (&colmask)[G],
+                                         int (&shift)[G], float (&scale)[G], float4v (&acc)[R][G]) {
+    half8v bhi[G], blo[G];
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        // Largest magnitude of this rhs column over the step's 32 columns (the 4 lanes that
+        // share the column hold 8 each).
+        float m = 0.0f;
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+            m = fmaxf(m, fabsf(raw[g][t] * keep[t]));
+        }
+        m = fmaxf(m, __shfl_xor(m, 16, 64));
+        m = fmaxf(m, __shfl_xor(m, 32, 64));
+        const bool grow = colmask[g] && !(m * scale[g] < 32768.0f);
+        if (__any(grow)) {
+            if (grow) {
+                // m < 2^e, so m * 2^(14 - e) < 2^14.
+                const int e = __builtin_amdgcn_frexp_expf(m);
+                const int new_shift = min(max(KM_F16_KSCALE_LOG2 - e, -100), 100);
+                const float factor = __builtin_ldexpf(1.0f, new_shift - shift[g]);
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    acc[r][g] *= factor;
+                }
+                shift[g] = new_shift;
+                scale[g] = __builtin_ldexpf(1.0f, new_shift);
+            }
+        }
+        float rv[8];
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+            rv[t] = raw[g][t] * (keep[t] * scale[g]);
+        }
+        split_f16x8(rv, &bhi[g], &blo[g]);
+    }
+
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        half8v ahi, alo;
+#pragma unroll
+        for (int t = 0; t < 8; t += 2) {
+            half2v h, l;
+            kernel_pair_f16<KT>(x1v[r], x2v[t], x2v[t + 1], kc, &h, &l);
+            ahi[t] = h[0];
+            ahi[t + 1] = h[1];
+            alo[t] = l[0];
+            alo[t + 1] = l[1];
+        }
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            acc[r][g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahi, bhi[g], acc[r][g], 0, 0, 0);
+            acc[r][g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahi, blo[g], acc[r][g], 0, 0, 0);
+            acc[r][g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(alo, bhi[g], acc[r][g], 0, 0, 0);
+        }
+    }
+}
+
 template <int KT, int G, int R>
 __global__ void __launch_bounds__(512) fwd_mfma_f16(const FwdArgs a) {
     extern __shared__ float lds[];
@@ -391,44 +456,21 @@ __global__ void __launch_bounds__(512) fwd_mfma_f16(const FwdArgs a) {
         x1v[r] = w.x1[(long long)row * a.x1_s];
     }
 
+    // rhs columns past k read a valid column instead and are zeroed through their scale.
     bool colmask[G];
+    unsigned rhs_lane[G];  // element offset of (column 8 kk, rhs column of this lane)
+    int shift[G];
+    float scale[G];
 #pragma unroll
     for (int g = 0; g < G; g++) {
-        colmask[g] = kbase + 16 * g + li < a.k;
+        const int c = kbase + 16 * g + li;
+        colmask[g] = c < a.k;
+        rhs_lane[g] = (unsigned)(8 * kk * a.rhs_s0 + min(c, a.k - 1) * a.rhs_s1);
+        // Start far up so that the first non-zero step sets the real scale.
+        shift[g] = 100;
+        scale[g] = colmask[g] ? __builtin_ldexpf(1.0f, 100) : 0.0f;
     }
-    const float* __restrict__ rhs_lane = w.rhs + (long long)(kbase + li) * a.rhs_s1;
-    const long long g_step = 16 * a.rhs_s1;
-
-    // Pre-scan: largest |rhs| per rhs column over this wavefront's window -> power-of-two scale
-    // that brings the column below 2^14.
-    float scale[G], unscale[G];
-    {
-        float cmax[G];
-#pragma unroll
-        for (int g = 0; g < G; g++) {
-            cmax[g] = 0.0f;
-        }
-        for (int col = col_begin + kk; col < col_end; col += 4) {
-            const float* p = rhs_lane + (long long)col * a.rhs_s0;
-#pragma unroll
-            for (int g = 0; g < G; g++) {
-                if (colmask[g]) {
-                    cmax[g] = fmaxf(cmax[g], fabsf(p[g * g_step]));
-                }
-            }
-        }
-#pragma unroll
-        for (int g = 0; g < G; g++) {
-            cmax[g] = fmaxf(cmax[g], __shfl_xor(cmax[g], 16, 64));
-            cmax[g] = fmaxf(cmax[g], __shfl_xor(cmax[g], 32, 64));
-            // cmax < 2^e  =>  cmax * 2^(14 - e) < 2^14; the shift is clamped so that the scale
-            // and its inverse stay normal numbers.
-            const int e = cmax[g] > 0.0f ? __builtin_amdgcn_frexp_expf(cmax[g]) : KM_F16_KSCALE_LOG2;
-            const int shift = min(max(KM_F16_KSCALE_LOG2 - e, -100), 100);
-            scale[g] = __builtin_ldexpf(1.0f, shift);
-            unscale[g] = __builtin_ldexpf(sigma, -shift - KM_F16_KSCALE_LOG2);
-        }
-    }
+    const unsigned x2_lane = (unsigned)(8 * kk * a.x2_s);
 
     float4v acc[R][G];
 #pragma unroll
@@ -439,56 +481,84 @@ __global__ void __launch_bounds__(512) fwd_mfma_f16(const FwdArgs a) {
         }
     }
 
-    const int last_col = a.n - 1;
-    for (int c0 = col_begin; c0 < col_end; c0 += 32) {
-        // This lane's 8 columns of the step.  Columns past the range keep a valid x2 (clamped
-        // index) and get a zero rhs operand.
-        const int cbase = c0 + 8 * kk;
-        float x2v[8];
-        half8v bhi[G], blo[G];
+    const float ones[8] = {1.0f, 1.0f, 1.0f, 1.0f, 1.0f, 1.0f, 1.0f, 1.0f};
+
+    // Full steps.  Addresses are a wave-uniform base (scalar registers, advanced once per
+    // step) plus a loop-invariant 32-bit lane offset; the next step's operands are requested
+    // before the current step is evaluated.
+    const int full_end = col_begin + ((max(col_end - col_begin, 0)) & ~31);
+    int c0 = col_begin;
+    if (c0 < full_end) {
+        const float* x2u = w.x2 + (long long)c0 * a.x2_s;
+        const float* ru = w.rhs + (long long)c0 * a.rhs_s0;
+        float x2v[8], raw[G][8];
 #pragma unroll
         for (int t = 0; t < 8; t++) {
-            x2v[t] = w.x2[(long long)min(cbase + t, last_col) * a.x2_s];
-        }
-#pragma unroll
-        for (int g = 0; g < G; g++) {
-            float rv[8];
-#pragma unroll
-            for (int t = 0; t < 8; t++) {
-                const int col = cbase + t;
-                rv[t] = (col < col_end && colmask[g])
-                            ? rhs_lane[(long long)col * a.rhs_s0 + g * g_step] * scale[g]
-                            : 0.0f;
-            }
-            split_f16x8(rv, &bhi[g], &blo[g]);
-        }
-
-#pragma unroll
-        for (int r = 0; r < R; r++) {
-            half8v ahi, alo;
-#pragma unroll
-            for (int t = 0; t < 8; t += 2) {
-                half2v h, l;
-                kernel_pair_f16<KT>(x1v[r], x2v[t], x2v[t + 1], kc, &h, &l);
-                ahi[t] = h[0];
-                ahi[t + 1] = h[1];
-                alo[t] = l[0];
-                alo[t + 1] = l[1];
-            }
+            x2v[t] = (x2u + t * a.x2_s)[x2_lane];
 #pragma unroll
             for (int g = 0; g < G; g++) {
-                acc[r][g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahi, bhi[g], acc[r][g], 0, 0, 0);
-                acc[r][g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahi, blo[g], acc[r][g], 0, 0, 0);
-                acc[r][g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(alo, bhi[g], acc[r][g], 0, 0, 0);
+                raw[g][t] = (ru + t * a.rhs_s0)[rhs_lane[g]];
+            }
+        }
+        for (; c0 < full_end; c0 += 32) {
+            x2u += 32 * a.x2_s;
+            ru += 32 * a.rhs_s0;
+            float x2n[8], rawn[G][8];
+            if (c0 + 32 < full_end) {
+#pragma unroll
+                for (int t = 0; t < 8; t++) {
+                    x2n[t] = (x2u + t * a.x2_s)[x2_lane];
+#pragma unroll
+                    for (int g = 0; g < G; g++) {
+                        rawn[g][t] = (ru + t * a.rhs_s0)[rhs_lane[g]];
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int t = 0; t < 8; t++) {
+                    x2n[t] = x2v[t];
+#pragma unroll
+                    for (int g = 0; g < G; g++) {
+                        rawn[g][t] = 0.0f;
+                    }
+                }
+            }
+            f16_step<KT, G, R>(x2v, raw, ones, x1v, kc, colmask, shift, scale, acc);
+#pragma unroll
+            for (int t = 0; t < 8; t++) {
+                x2v[t] = x2n[t];
+#pragma unroll
+                for (int g = 0; g < G; g++) {
+                    raw[g][t] = rawn[g][t];
+                }
             }
         }
     }
 
+    // Partial last step: columns past the range read the last valid column and are dropped
+    // through a zero factor.
+    if (c0 < col_end) {
+        float x2v[8], raw[G][8], keep[8];
 #pragma unroll
-    for (int r = 0; r < R; r++) {
+        for (int t = 0; t < 8; t++) {
+            const int col = c0 + 8 * kk + t;
+            const int colc = min(col, col_end - 1);
+            keep[t] = col < col_end ? 1.0f : 0.0f;
+            x2v[t] = w.x2[(long long)colc * a.x2_s];
 #pragma unroll
-        for (int g = 0; g < G; g++) {
-            acc[r][g] *= unscale[g];
+            for (int g = 0; g < G; g++) {
+                raw[g][t] = w.rhs[(long long)colc * a.rhs_s0 + (rhs_lane[g] - (unsigned)(8 * kk * a.rhs_s0))];
+            }
+        }
+        f16_step<KT, G, R>(x2v, raw, keep, x1v, kc, colmask, shift, scale, acc);
+    }
+
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        const float unscale = __builtin_ldexpf(sigma, -shift[g] - KM_F16_KSCALE_LOG2);
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            acc[r][g] *= unscale;
         }
     }
     float* __restrict__ out = a.out + w.b * (long long)a.m * a.k;
