@@ -124,6 +124,14 @@ static int make_plan(const MatmulProblem& p, const km_launch_options* opt, Matmu
             S *= 2;
         }
     }
+    // Register budget of the split-fp16 kernel: its operand buffers grow with G, so wide rhs
+    // tiles get fewer row groups per wavefront (no spills, at least two wavefronts per SIMD).
+    if (variant == KM_VARIANT_MFMA_F16) {
+        const int max_r = G == 1 ? 8 : (G == 2 ? 4 : 2);
+        if (R > max_r) {
+            R = max_r;
+        }
+    }
     // The cross-wavefront reduction buffer (S * R * G KiB) must fit 64 KiB of LDS.
     while (S > 1 && S * R * G > 64) {
         S /= 2;

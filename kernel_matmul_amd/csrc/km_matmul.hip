@@ -353,14 +353,48 @@ __device__ __forceinline__ void split_f16x8(const float (&v)[8], half8v* hi, hal
     }
 }
 
+// Operands of one step of 32 columns for this lane: x2 and rhs at columns c0 + 8 kk + t.
+// Full steps use a wave-uniform base (scalar registers) plus a loop-invariant 32-bit lane
+// offset; the partial last step clamps the column to the range and zeroes the rhs operand of
+// columns past it.
+template <int G>
+__device__ __forceinline__ void f16_load(const FwdArgs& a, const WaveView& w, int c0, int col_end,
+                                         int kk, unsigned x2_lane, const unsigned (&rhs_lane)[G],
+                                         float (&x2v)[8], float (&raw)[G][8]) {
+    if (c0 + 32 <= col_end) {
+        const float* x2u = w.x2 + (long long)c0 * a.x2_s;
+        const float* ru = w.rhs + (long long)c0 * a.rhs_s0;
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+            x2v[t] = (x2u + t * a.x2_s)[x2_lane];
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                raw[g][t] = (ru + t * a.rhs_s0)[rhs_lane[g]];
+            }
+        }
+    } else {
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+            const int col = c0 + 8 * kk + t;
+            const int colc = min(col, col_end - 1);
+            x2v[t] = w.x2[(long long)colc * a.x2_s];
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                const float v = w.rhs[(long long)colc * a.rhs_s0 + (rhs_lane[g] - (unsigned)(8 * kk * a.rhs_s0))];
+                raw[g][t] = col < col_end ? v : 0.0f;
+            }
+        }
+    }
+}
+
 // One step of 32 columns: convert this lane's 8 rhs values per column group to hi/lo halves
 // (rescaling the accumulators first if a value would leave the fp16 range), then for every
 // row group evaluate 8 kernel entries, split them and issue the three MFMAs.
 template <int KT, int G, int R>
 __device__ __forceinline__ void f16_step(const float (&x2v)[8], const float (&raw)[G][8],
-                                         const float (&keep)[8], const float (&x1v)[R],
-                                         const KernelConsts& kc, const bool (&colmask)[G],
-                                         int (&shift)[G], float (&scale)[G], float4v (&acc)[R][G]) {
+                                         const float (&x1v)[R], const KernelConsts& kc,
+                                         const bool (&colmask)[G], int (&shift)[G],
+                                         float (&scale)[G], float4v (&acc)[R][G]) {
     half8v bhi[G], blo[G];
 #pragma unroll
     for (int g = 0; g < G; g++) {
@@ -369,7 +403,7 @@ __device__ __forceinline__ void f16_step(const float (&x2v)[8], const float (&ra
         float m = 0.0f;
 #pragma unroll
         for (int t = 0; t < 8; t++) {
-            m = fmaxf(m, fabsf(raw[g][t] * keep[t]));
+            m = fmaxf(m, fabsf(raw[g][t]));
         }
         m = fmaxf(m, __shfl_xor(m, 16, 64));
         m = fmaxf(m, __shfl_xor(m, 32, 64));
@@ -391,7 +425,7 @@ __device__ __forceinline__ void f16_step(const float (&x2v)[8], const float (&ra
         float rv[8];
 #pragma unroll
         for (int t = 0; t < 8; t++) {
-            rv[t] = raw[g][t] * (keep[t] * scale[g]);
+            rv[t] = raw[g][t] * scale[g];
         }
         split_f16x8(rv, &bhi[g], &blo[g]);
     }
@@ -417,7 +451,9 @@ __device__ __forceinline__ void f16_step(const float (&x2v)[8], const float (&ra
     }
 }
 
-template <int KT, int G, int R>
+// PF: request the next step's operands before evaluating the current one (costs 8 + 8 G
+// registers; used for G = 1 where they are available).
+template <int KT, int G, int R, bool PF>
 __global__ void __launch_bounds__(512) fwd_mfma_f16(const FwdArgs a) {
     extern __shared__ float lds[];
 
@@ -481,76 +517,34 @@ __global__ void __launch_bounds__(512) fwd_mfma_f16(const FwdArgs a) {
         }
     }
 
-    const float ones[8] = {1.0f, 1.0f, 1.0f, 1.0f, 1.0f, 1.0f, 1.0f, 1.0f};
-
-    // Full steps.  Addresses are a wave-uniform base (scalar registers, advanced once per
-    // step) plus a loop-invariant 32-bit lane offset; the next step's operands are requested
-    // before the current step is evaluated.
-    const int full_end = col_begin + ((max(col_end - col_begin, 0)) & ~31);
-    int c0 = col_begin;
-    if (c0 < full_end) {
-        const float* x2u = w.x2 + (long long)c0 * a.x2_s;
-        const float* ru = w.rhs + (long long)c0 * a.rhs_s0;
+    if (col_begin < col_end) {
         float x2v[8], raw[G][8];
+        f16_load<G>(a, w, col_begin, col_end, kk, x2_lane, rhs_lane, x2v, raw);
+        for (int c0 = col_begin; c0 < col_end; c0 += 32) {
+            const bool more = c0 + 32 < col_end;
+            if (PF) {
+                float x2n[8], rawn[G][8];
+                if (more) {
+                    f16_load<G>(a, w, c0 + 32, col_end, kk, x2_lane, rhs_lane, x2n, rawn);
+                }
+                f16_step<KT, G, R>(x2v, raw, x1v, kc, colmask, shift, scale, acc);
+                if (more) {
 #pragma unroll
-        for (int t = 0; t < 8; t++) {
-            x2v[t] = (x2u + t * a.x2_s)[x2_lane];
+                    for (int t = 0; t < 8; t++) {
+                        x2v[t] = x2n[t];
 #pragma unroll
-            for (int g = 0; g < G; g++) {
-                raw[g][t] = (ru + t * a.rhs_s0)[rhs_lane[g]];
-            }
-        }
-        for (; c0 < full_end; c0 += 32) {
-            x2u += 32 * a.x2_s;
-            ru += 32 * a.rhs_s0;
-            float x2n[8], rawn[G][8];
-            if (c0 + 32 < full_end) {
-#pragma unroll
-                for (int t = 0; t < 8; t++) {
-                    x2n[t] = (x2u + t * a.x2_s)[x2_lane];
-#pragma unroll
-                    for (int g = 0; g < G; g++) {
-                        rawn[g][t] = (ru + t * a.rhs_s0)[rhs_lane[g]];
+                        for (int g = 0; g < G; g++) {
+                            raw[g][t] = rawn[g][t];
+                        }
                     }
                 }
             } else {
-#pragma unroll
-                for (int t = 0; t < 8; t++) {
-                    x2n[t] = x2v[t];
-#pragma unroll
-                    for (int g = 0; g < G; g++) {
-                        rawn[g][t] = 0.0f;
-                    }
-                }
-            }
-            f16_step<KT, G, R>(x2v, raw, ones, x1v, kc, colmask, shift, scale, acc);
-#pragma unroll
-            for (int t = 0; t < 8; t++) {
-                x2v[t] = x2n[t];
-#pragma unroll
-                for (int g = 0; g < G; g++) {
-                    raw[g][t] = rawn[g][t];
+                f16_step<KT, G, R>(x2v, raw, x1v, kc, colmask, shift, scale, acc);
+                if (more) {
+                    f16_load<G>(a, w, c0 + 32, col_end, kk, x2_lane, rhs_lane, x2v, raw);
                 }
             }
         }
-    }
-
-    // Partial last step: columns past the range read the last valid column and are dropped
-    // through a zero factor.
-    if (c0 < col_end) {
-        float x2v[8], raw[G][8], keep[8];
-#pragma unroll
-        for (int t = 0; t < 8; t++) {
-            const int col = c0 + 8 * kk + t;
-            const int colc = min(col, col_end - 1);
-            keep[t] = col < col_end ? 1.0f : 0.0f;
-            x2v[t] = w.x2[(long long)colc * a.x2_s];
-#pragma unroll
-            for (int g = 0; g < G; g++) {
-                raw[g][t] = w.rhs[(long long)colc * a.rhs_s0 + (rhs_lane[g] - (unsigned)(8 * kk * a.rhs_s0))];
-            }
-        }
-        f16_step<KT, G, R>(x2v, raw, keep, x1v, kc, colmask, shift, scale, acc);
     }
 
 #pragma unroll
@@ -637,7 +631,7 @@ static hipError_t launch_mfma(const FwdArgs& a, int variant, int S, unsigned gx,
                               hipStream_t stream) {
     const size_t lds = S > 1 ? (size_t)S * R * G * 4 * 64 * sizeof(float) : 0;
     if (variant == KM_VARIANT_MFMA_F16) {
-        hipLaunchKernelGGL((fwd_mfma_f16<KT, G, R>), dim3(gx, gy, 1), dim3(64 * S, 1, 1), lds, stream, a);
+        hipLaunchKernelGGL((fwd_mfma_f16<KT, G, R, G == 1>), dim3(gx, gy, 1), dim3(64 * S, 1, 1), lds, stream, a);
     } else {
         hipLaunchKernelGGL((fwd_mfma_f32<KT, G, R>), dim3(gx, gy, 1), dim3(64 * S, 1, 1), lds, stream, a);
     }
