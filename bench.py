@@ -36,6 +36,9 @@ WORKLOADS = {
                label="spectral K@rhs n=1000000 k=32 batch=8 cutoff=5*l_max"),
 }
 
+# (FETCH_SIZE 3543.6 KiB x 2.00 + WRITE_SIZE 50000.0 KiB x 1.00) x 1024
+MEASURED_TRAFFIC_BYTES = {"headline": 58457292}
+
 FLOPS_PER_PAIR = {"rbf": lambda k: 5 + 2 * k, "spectral": lambda k: 8 + 2 * k,
                   "locally_periodic": lambda k: 10 + 2 * k}
 
@@ -73,6 +76,9 @@ def main() -> int:
     ap.add_argument("--col-splits", type=int, default=0)
     ap.add_argument("--batch", type=int, default=None, help="override the number of batch items")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 256 MiB elementwise add-scalar (a copy-like kernel of known traffic "
+                         "against which FETCH_SIZE / WRITE_SIZE counters are scaled)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     args = ap.parse_args()
 
@@ -127,6 +133,13 @@ def main() -> int:
     for _ in range(args.warmup):
         out = op.call(*op_args)
     torch.cuda.synchronize()
+    if args.calibrate_copy:
+        src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device=device)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        torch.add(src, 1.0, out=dst)  # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
 
     # Whole-step wall time and, on the launch stream, per-launch event time of the kernel.
     events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
@@ -147,11 +160,11 @@ def main() -> int:
     value = pairs / (ms_per_step * 1e-3)
     achieved_tflops = pairs * flops_per_pair / (kernel_ms_avg * 1e-3) / 1e12
 
+    # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
+    # profiles/fwd_mfma_f16_headline_counters.md (only measured for the default headline run).
     traffic = None
-    traffic_path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
-    if os.path.exists(traffic_path):
-        with open(traffic_path) as f:
-            traffic = json.load(f).get(args.workload, {}).get("bytes_per_launch")
+    if args.workload == "headline" and args.batch is None and args.variant in ("auto", "mfma_f16"):
+        traffic = MEASURED_TRAFFIC_BYTES["headline"]
 
     result = {
         "metric": "kernel-pair evaluations/s (sparse spectral K@rhs, n=100k, k=16, 1 MI355X)",
