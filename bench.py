@@ -32,6 +32,10 @@ WORKLOADS = {
                label="rbf K@rhs n=4096 k=1 l=sigma=1 cutoff=8"),
     "c2": dict(kernel="spectral", n=20_000, extent=2000.0, batch=4, k=16, cutoff_l=6.0, seed=1002,
                label="spectral K@rhs n=20000 k=16 batch=4 cutoff=6*l_max"),
+    "c3": dict(kernel="spectral", n=50_000, extent=None, batch=2, k=8, cutoff_l=6.0, seed=1003, op="param_grad",
+               label="spectral matmul_bwd n=50000 k=8 batch=2 x=cumsum(Exp(1)) cutoff=6*l_max"),
+    "c4": dict(kernel="spectral", n=100_000, extent=10_000.0, batch=16, k=4, cutoff_l=6.0, seed=1004, op="param_grad",
+               label="spectral bilinear_derivative n=100000 d=4 batch=16 cutoff=6*l_max"),
     "c5": dict(kernel="spectral", n=1_000_000, extent=100_000.0, batch=8, k=32, cutoff_l=5.0, seed=1005,
                label="spectral K@rhs n=1000000 k=32 batch=8 cutoff=5*l_max"),
 }
@@ -41,6 +45,7 @@ MEASURED_TRAFFIC_BYTES = {"headline": 58457292}
 
 FLOPS_PER_PAIR = {"rbf": lambda k: 5 + 2 * k, "spectral": lambda k: 8 + 2 * k,
                   "locally_periodic": lambda k: 10 + 2 * k}
+GRAD_FLOPS_PER_PAIR = {"rbf": lambda c: 6 + 2 * c + 2 * 2, "spectral": lambda c: 14 + 2 * c + 2 * 3}
 
 
 def make_workload(name: str, batch_override=None):
@@ -53,7 +58,10 @@ def make_workload(name: str, batch_override=None):
         w["label"] += f" [batch overridden to {batch_override}]"
     g = torch.Generator().manual_seed(w["seed"])
     n, batch = w["n"], w["batch"]
-    x = torch.sort(torch.rand(n, generator=g) * w["extent"])[0]
+    if w["extent"] is None:  # irregular grid: cumulative sum of Exp(1) gaps
+        x = torch.cumsum(-torch.log1p(-torch.rand(n, generator=g)), dim=0)
+    else:
+        x = torch.sort(torch.rand(n, generator=g) * w["extent"])[0]
     bshape = (batch,) if batch else ()
     u = lambda lo, hi: lo + (hi - lo) * torch.rand(bshape, generator=g)
     if w["kernel"] == "spectral":
@@ -108,7 +116,8 @@ def main() -> int:
     rows_in_block = torch.clamp(n - 128 * torch.arange(row_blocks), max=128)
     pairs_per_item = int((rows_in_block * (end_cpu - start_cpu)).sum())
     pairs = pairs_per_item * max(batch, 1)
-    flops_per_pair = FLOPS_PER_PAIR[w["kernel"]](k)
+    is_grad = w.get("op") == "param_grad"
+    flops_per_pair = (GRAD_FLOPS_PER_PAIR if is_grad else FLOPS_PER_PAIR)[w["kernel"]](k)
 
     x = x_cpu.to(device)
     rhs = rhs_cpu.to(device)
@@ -129,6 +138,14 @@ def main() -> int:
     if args.col_splits:
         defines["MATMUL_COL_BLOCKS"] = args.col_splits
     op = load_native("matmul", defines)
+    if is_grad:
+        from kernel_matmul_amd.configurations import BilinearDerivativeConfiguration
+
+        g2 = torch.Generator().manual_seed(w["seed"] + 50)
+        left = torch.randn(n, k, generator=g2).to(device).expand(*bshape, n, k)
+        op_args = (xb, xb, left, rhsb, params, startb, endb)
+        op = load_native("bilinear_derivative",
+                         BilinearDerivativeConfiguration(w["kernel"]).make_config(op_args))
 
     for _ in range(args.warmup):
         out = op.call(*op_args)
@@ -188,7 +205,7 @@ def main() -> int:
         },
         "roofline": {
             "bound": "mfma",
-            "kernel": {"auto": "km::fwd_mfma_f16", "mfma_f16": "km::fwd_mfma_f16", "mfma_f32": "km::fwd_mfma_f32", "valu": "km::fwd_valu"}[args.variant],
+            "kernel": "km::param_grad_partial" if is_grad else {"auto": "km::fwd_mfma_f16", "mfma_f16": "km::fwd_mfma_f16", "mfma_f32": "km::fwd_mfma_f32", "valu": "km::fwd_valu"}[args.variant],
             "achieved": achieved_tflops,
             "peak": PEAK_FP32_TFLOPS,
             "unit": "TFLOP/s",
@@ -202,7 +219,7 @@ def main() -> int:
         },
     }
 
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and not is_grad:
         from oracle import dense_cpu
 
         p0 = params_cpu[0] if batch else params_cpu

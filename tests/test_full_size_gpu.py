@@ -1,0 +1,188 @@
+"""Parity at the full BASELINE.json sizes through properties that do not need a dense oracle:
+oracle on sampled row blocks, linearity in rhs, symmetry of the bilinear form, agreement of the
+three contraction variants, d/d(outputscale) identity, index lookups against per-entry closed
+forms, and bit-exact device ranges at n = 10^6."""
+import zlib
+
+import numpy as np
+import pytest
+import torch
+
+from kernel_matmul_amd.compile import load_native
+from kernel_matmul_amd.configurations import (
+    BilinearDerivativeConfiguration,
+    IndexConfiguration,
+    MatmulBwdConfiguration,
+    MatmulSingleConfiguration,
+)
+from kernel_matmul_amd.ranges import make_ranges
+from oracle import kernels as oracle
+from oracle import ranges as oracle_ranges
+
+pytestmark = pytest.mark.gpu
+
+CONFIGS = {
+    # name: kernel, n, extent (None = cumulative Exp(1) gaps), batch, k, cutoff factor
+    "c2": ("spectral", 20_000, 2000.0, 4, 16, 6.0),
+    "c3": ("spectral", 50_000, None, 2, 8, 6.0),
+    "c3_rbf": ("rbf", 50_000, None, 2, 8, 6.0),
+    "headline": ("spectral", 100_000, 10_000.0, 8, 16, 6.0),
+    "c5": ("spectral", 1_000_000, 100_000.0, 8, 32, 5.0),
+}
+
+
+def _build(name):
+    kernel, n, extent, batch, k, cf = CONFIGS[name]
+    g = torch.Generator().manual_seed(zlib.crc32(name.encode()) % 1000 + 2000)
+    if extent is None:
+        x = torch.cumsum(-torch.log1p(-torch.rand(n, generator=g)), dim=0)
+    else:
+        x = torch.sort(torch.rand(n, generator=g) * extent)[0]
+    u = lambda lo, hi: lo + (hi - lo) * torch.rand(batch, generator=g)
+    if kernel == "spectral":
+        params = torch.stack([u(0.5, 2.0), u(0.05, 0.5), u(0.5, 2.0)], dim=-1)
+    else:
+        params = torch.stack([u(0.5, 2.0), u(0.5, 2.0)], dim=-1)
+    rhs = torch.randn(n, k, generator=g)
+    cutoff = cf * float(params[:, 0].max())
+    device = torch.device("cuda:0")
+    xd = x.to(device)
+    start, end = make_ranges(cutoff, xd)
+    rows = start.shape[-1]
+    args = dict(
+        x=xd.expand(batch, n), rhs=rhs.to(device).expand(batch, n, k), params=params.to(device),
+        start=start.expand(batch, rows), end=end.expand(batch, rows),
+    )
+    host = dict(x=x.numpy(), rhs=rhs.numpy(), params=params.numpy(), start=start.cpu().numpy(),
+                end=end.cpu().numpy(), cutoff=cutoff)
+    return kernel, n, batch, k, args, host
+
+
+def _matmul(kernel, a, rhs=None, variant=None):
+    rhs = a["rhs"] if rhs is None else rhs
+    op_args = (a["x"], a["x"], rhs, a["params"], a["start"], a["end"])
+    defines = MatmulSingleConfiguration(kernel).make_config(op_args)
+    if variant:
+        defines["MATMUL_VARIANT"] = variant
+    return load_native("matmul", defines).call(*op_args)
+
+
+@pytest.mark.parametrize("name", ["c2", "c3_rbf", "headline", "c5"])
+def test_forward_sampled_blocks_against_oracle(name):
+    kernel, n, batch, k, a, h = _build(name)
+    out = _matmul(kernel, a)
+    assert out.shape == (batch, n, k)
+    blocks = np.unique(np.concatenate([[0, 1, len(h["start"]) - 1],
+                                       np.random.default_rng(1).integers(0, len(h["start"]), 5)]))
+    for blk in blocks:
+        r0, r1 = blk * 128, min(blk * 128 + 128, n)
+        s, e = int(h["start"][blk]), int(h["end"][blk])
+        x1 = np.broadcast_to(h["x"][r0:r1], (batch, r1 - r0))
+        x2 = np.broadcast_to(h["x"][s:e], (batch, e - s))
+        rhs = np.broadcast_to(h["rhs"][s:e], (batch, e - s, k))
+        full = np.zeros((batch, 1), dtype=np.int64)
+        expected = oracle.matmul(kernel, x1, x2, rhs, h["params"], full, full + (e - s))
+        got = out[:, r0:r1].cpu().double().numpy()
+        err = np.abs(got - expected)
+        assert np.all(err <= 1e-5 + 1e-4 * np.abs(expected)), (name, blk, err.max())
+
+
+@pytest.mark.parametrize("name", ["headline", "c5"])
+def test_forward_linearity_symmetry_and_variants(name):
+    kernel, n, batch, k, a, h = _build(name)
+    out = _matmul(kernel, a)
+    scale = out.abs().mean()
+
+    # linear in rhs
+    g = torch.Generator().manual_seed(3)
+    other = torch.randn(n, k, generator=g).to(out.device).expand(batch, n, k)
+    mixed = _matmul(kernel, a, rhs=1.5 * a["rhs"] - 0.25 * other)
+    expected = 1.5 * out - 0.25 * _matmul(kernel, a, rhs=other)
+    assert torch.allclose(mixed, expected, rtol=1e-4, atol=float(1e-4 * scale))
+
+    # K is symmetric on the symmetric pattern: <u, K v> == <v, K u>
+    lhs = (other * out).double().sum(dim=(-2, -1))
+    rhs_side = (a["rhs"] * _matmul(kernel, a, rhs=other)).double().sum(dim=(-2, -1))
+    denom = (other.double().norm() * out.double().norm() / batch**0.5)
+    assert torch.all((lhs - rhs_side).abs() <= 1e-5 * denom)
+
+    # the three contraction variants agree
+    for variant in ("mfma_f32", "valu"):
+        alt = _matmul(kernel, a, variant=variant)
+        assert torch.allclose(alt, out, rtol=1e-4, atol=float(1e-4 * scale)), variant
+
+
+@pytest.mark.parametrize("name", ["c3", "c3_rbf", "headline"])
+def test_param_grad_identities(name):
+    kernel, n, batch, k, a, h = _build(name)
+    g = torch.Generator().manual_seed(4)
+    grad_out = torch.randn(batch, n, k, generator=g).to(a["x"].device)
+    bwd_args = (a["x"], a["x"], a["rhs"], a["params"], a["start"], a["end"], grad_out)
+    bwd = load_native("matmul_bwd", MatmulBwdConfiguration(kernel).make_config(bwd_args)).call(*bwd_args)
+    bil_args = (a["x"], a["x"], grad_out, a["rhs"], a["params"], a["start"], a["end"])
+    bil = load_native("bilinear_derivative",
+                      BilinearDerivativeConfiguration(kernel).make_config(bil_args)).call(*bil_args)
+    assert torch.equal(bwd, bil)  # same sum, same kernel, fixed reduction order
+    again = load_native("matmul_bwd", MatmulBwdConfiguration(kernel).make_config(bwd_args)).call(*bwd_args)
+    assert torch.equal(bwd, again)  # run-to-run reproducible
+
+    # d/d(outputscale) = <grad_out, K rhs> / outputscale
+    out = _matmul(kernel, a)
+    expected = (grad_out.double() * out.double()).sum(dim=(-2, -1)) / a["params"][:, -1].double()
+    ref_scale = (grad_out.double().norm(dim=(-2, -1)) * out.double().norm(dim=(-2, -1))) / a["params"][:, -1].double()
+    assert torch.all((bwd[:, -1].double() - expected).abs() <= 1e-5 * ref_scale + 1e-4 * expected.abs())
+
+    # oracle on a sub-problem: the rows of a few row blocks only
+    nblk = len(h["start"])
+    for blk in (0, nblk // 2, nblk - 1):
+        r0, r1 = blk * 128, min(blk * 128 + 128, n)
+        s, e = int(h["start"][blk]), int(h["end"][blk])
+        sub = dict(x1=a["x"][:, r0:r1], left=grad_out[:, r0:r1])
+        zeros = torch.zeros(batch, 1, dtype=torch.int32, device=a["x"].device)
+        sub_args = (sub["x1"], a["x"][:, s:e], sub["left"], a["rhs"][:, s:e], a["params"], zeros, zeros + (e - s))
+        got = load_native("bilinear_derivative",
+                          BilinearDerivativeConfiguration(kernel).make_config(sub_args)).call(*sub_args)
+        expected = oracle.param_grad(
+            kernel, np.broadcast_to(h["x"][r0:r1], (batch, r1 - r0)), np.broadcast_to(h["x"][s:e], (batch, e - s)),
+            grad_out[:, r0:r1].cpu().numpy(), np.broadcast_to(h["rhs"][s:e], (batch, e - s, k)), h["params"],
+            np.zeros((batch, 1), dtype=np.int64), np.full((batch, 1), e - s))
+        tol = 1e-5 + 1e-4 * np.abs(expected).max(axis=-1, keepdims=True)
+        assert np.all(np.abs(got.cpu().double().numpy() - expected) <= tol), (name, blk)
+
+
+def test_index_rows_at_full_size():
+    kernel, n, batch, k, a, h = _build("c5")
+    rng = np.random.default_rng(9)
+    rows = rng.integers(0, n, 4096)
+    delta = rng.integers(-600, 600, 4096)
+    cols = np.clip(rows + delta, 0, n - 1)
+    bi = rng.integers(0, batch, 4096)
+    device = a["x"].device
+    t = lambda v: torch.from_numpy(v.astype(np.int32)).to(device)
+    args = (a["x"], a["x"], a["params"], a["start"], a["end"], (t(bi),), t(rows), t(cols))
+    got = load_native("index", IndexConfiguration(kernel).make_config(args)).call(*args)
+    blk = rows // 128
+    inside = (cols >= h["start"][blk]) & (cols < h["end"][blk])
+    assert 0 < inside.sum() < 4096
+    x = h["x"].astype(np.float64)
+    p = h["params"].astype(np.float64)[bi]
+    d = x[rows] - x[cols]
+    expected = np.where(inside, p[:, 2] * np.exp(-d * d / (2 * p[:, 0] ** 2)) * np.cos(2 * np.pi * p[:, 1] * d), 0.0)
+    np.testing.assert_allclose(got.cpu().double().numpy(), expected, rtol=1e-4, atol=1e-5)
+    assert torch.all(got[torch.from_numpy(~inside).to(device)] == 0)
+
+
+def test_ranges_at_full_size_bit_exact():
+    _, n, _, _, a, h = _build("c5")
+    s_ref, e_ref = oracle_ranges.make_ranges(h["cutoff"], h["x"])
+    np.testing.assert_array_equal(h["start"], s_ref)
+    np.testing.assert_array_equal(h["end"], e_ref)
+    x_cpu = torch.from_numpy(h["x"])
+    s_host, e_host = make_ranges(h["cutoff"], x_cpu)
+    np.testing.assert_array_equal(s_host.numpy(), s_ref)
+    x2 = x_cpu[::2].contiguous() + 0.003
+    for align in (False, True):
+        s_dev, e_dev = make_ranges(h["cutoff"], x_cpu.cuda(), x2.cuda(), align=align)
+        s_o, e_o = oracle_ranges.make_ranges(h["cutoff"], h["x"], x2.numpy(), align=align)
+        np.testing.assert_array_equal(s_dev.cpu().numpy(), s_o)
+        np.testing.assert_array_equal(e_dev.cpu().numpy(), e_o)
