@@ -152,6 +152,51 @@ int km_index(int kernel_type, int batch_rank, const int64_t* batch_sizes, int64_
              const int32_t* col_index, const int64_t* col_index_strides, float* out,
              void* stream);
 
+/* ------------------------------------------------------------------------------------
+ * index_bwd.  grad[b,p] = d/d params[b,p] sum_{q : batch(q) = b} out_grad[q] * K-entry(q)
+ * with the entries addressed exactly as in km_index; out_grad has the index shape.
+ * Replaces `call` of module km___index_bwd___* (native/index_bwd/index_bwd.cpp,
+ * native/index_bwd/index_bwd.cu:12-112).  grad[batch..., P] contiguous; `workspace` of at
+ * least km_index_bwd_workspace_size(number of index entries) bytes, contents irrelevant.
+ * ---------------------------------------------------------------------------------- */
+size_t km_index_bwd_workspace_size(int64_t num_entries);
+
+int km_index_bwd(int kernel_type, int batch_rank, const int64_t* batch_sizes, int64_t m, int64_t n,
+                 const float* x1, const int64_t* x1_strides, const float* x2,
+                 const int64_t* x2_strides, const float* params, const int64_t* params_strides,
+                 const int32_t* start, const int64_t* start_strides, const int32_t* end,
+                 const int64_t* end_strides, int index_rank, const int64_t* index_sizes,
+                 const int32_t* const* batch_index, const int64_t* const* batch_index_strides,
+                 const int32_t* row_index, const int64_t* row_index_strides,
+                 const int32_t* col_index, const int64_t* col_index_strides,
+                 const float* out_grad, const int64_t* out_grad_strides, float* grad,
+                 void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------
+ * dense.  out[b,i,j] = K[b,i,j] for j in the row block's [start, end), 0 elsewhere;
+ * out[batch..., m, n] contiguous and fully written.  Replaces `call` of module
+ * km___dense___* (native/dense/dense.cpp, native/dense/dense.cu:12-98).
+ * ---------------------------------------------------------------------------------- */
+int km_dense(int kernel_type, int batch_rank, const int64_t* batch_sizes, int64_t m, int64_t n,
+             const float* x1, const int64_t* x1_strides, const float* x2,
+             const int64_t* x2_strides, const float* params, const int64_t* params_strides,
+             const int32_t* start, const int64_t* start_strides, const int32_t* end,
+             const int64_t* end_strides, float* out, void* stream);
+
+/* ------------------------------------------------------------------------------------
+ * dense_bwd.  grad[b,p] = d/d params[b,p] sum_{(i,j) in mask} out_grad[b,i,j] K[b,i,j].
+ * Replaces `call` of module km___dense_bwd___* (native/dense_bwd/dense_bwd.cpp,
+ * native/dense_bwd/dense_bwd.cu:12-116).  out_grad[batch..., m, n] with strides;
+ * grad[batch..., P] contiguous; workspace as for km_param_grad (same size function).
+ * ---------------------------------------------------------------------------------- */
+int km_dense_bwd(int kernel_type, int batch_rank, const int64_t* batch_sizes, int64_t m, int64_t n,
+                 const float* x1, const int64_t* x1_strides, const float* x2,
+                 const int64_t* x2_strides, const float* params, const int64_t* params_strides,
+                 const int32_t* start, const int64_t* start_strides, const int32_t* end,
+                 const int64_t* end_strides, const float* out_grad,
+                 const int64_t* out_grad_strides, float* grad, void* workspace,
+                 size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

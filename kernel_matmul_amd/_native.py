@@ -100,6 +100,26 @@ def load_library():
         + tensor * 2
         + [_vp, _vp]
     )
+    lib.km_index_bwd_workspace_size.restype = ctypes.c_size_t
+    lib.km_index_bwd_workspace_size.argtypes = [ctypes.c_int64]
+    lib.km_index_bwd.restype = ctypes.c_int
+    lib.km_index_bwd.argtypes = (
+        [ctypes.c_int, ctypes.c_int, _i64p, ctypes.c_int64, ctypes.c_int64]
+        + tensor * 5
+        + [ctypes.c_int, _i64p, ctypes.POINTER(_vp), ctypes.POINTER(_i64p)]
+        + tensor * 3
+        + [_vp, _vp, ctypes.c_size_t, _vp]
+    )
+    lib.km_dense.restype = ctypes.c_int
+    lib.km_dense.argtypes = (
+        [ctypes.c_int, ctypes.c_int, _i64p, ctypes.c_int64, ctypes.c_int64] + tensor * 5 + [_vp, _vp]
+    )
+    lib.km_dense_bwd.restype = ctypes.c_int
+    lib.km_dense_bwd.argtypes = (
+        [ctypes.c_int, ctypes.c_int, _i64p, ctypes.c_int64, ctypes.c_int64]
+        + tensor * 6
+        + [_vp, _vp, ctypes.c_size_t, _vp]
+    )
     _lib = lib
     return lib
 
@@ -273,9 +293,7 @@ def index(kernel_type: str, x1: Tensor, x2: Tensor, params: Tensor, start: Tenso
     lib = load_library()
     out = torch.empty(shape, dtype=torch.float32, device=x1.device)
     rank = len(batch_shape)
-    bi_ptrs = (_vp * max(rank, 1))(*[t.data_ptr() for t in batch_indices])
-    bi_stride_arrays = [_i64(t.stride()) for t in batch_indices]
-    bi_strides = (_i64p * max(rank, 1))(*[ctypes.cast(a, _i64p) for a in bi_stride_arrays])
+    bi_ptrs, bi_strides, _keep = _batch_index_args(batch_indices, rank)
     with torch.cuda.device(x1.device):
         status = lib.km_index(
             kid, rank, _i64(batch_shape), x1.shape[-1], x2.shape[-1],
@@ -287,6 +305,102 @@ def index(kernel_type: str, x1: Tensor, x2: Tensor, params: Tensor, start: Tenso
     if status != 0:
         _raise(lib, status)
     return out
+
+
+def _batch_index_args(batch_indices, rank):
+    bi_ptrs = (_vp * max(rank, 1))(*[t.data_ptr() for t in batch_indices])
+    stride_arrays = [_i64(t.stride()) for t in batch_indices]
+    bi_strides = (_i64p * max(rank, 1))(*[ctypes.cast(a, _i64p) for a in stride_arrays])
+    return bi_ptrs, bi_strides, stride_arrays  # the arrays must outlive the call
+
+
+def index_bwd(kernel_type: str, x1: Tensor, x2: Tensor, params: Tensor, start: Tensor, end: Tensor,
+              batch_indices: Sequence[Tensor], row_index: Tensor, col_index: Tensor,
+              out_grad: Tensor) -> Tensor:
+    """grad[..., P] of sum(out_grad * index(...)) w.r.t. params   (C ABI: km_index_bwd)."""
+    kid = _kernel_id(kernel_type)
+    batch_shape = _check_matrix_inputs(kernel_type, x1, x2, params, start, end)
+    batch_indices = tuple(batch_indices)
+    if len(batch_indices) != len(batch_shape):
+        raise RuntimeError(
+            f"expected {len(batch_shape)} batch index tensors, got {len(batch_indices)}"
+        )
+    for t in (*batch_indices, row_index, col_index):
+        check_cuda_int32(t)
+    check_cuda(out_grad)
+    check_float(out_grad)
+    if row_index.dim() == 0:
+        return index_bwd(kernel_type, x1, x2, params, start, end,
+                         [b.reshape(1) for b in batch_indices], row_index.reshape(1),
+                         col_index.reshape(1), out_grad.reshape(1))
+    shape = tuple(row_index.shape)
+    for t in (*batch_indices, col_index, out_grad):
+        if tuple(t.shape) != shape:
+            raise RuntimeError("all index tensors and out_grad must have the same shape")
+    lib = load_library()
+    rank = len(batch_shape)
+    grad = torch.empty((*batch_shape, params.shape[-1]), dtype=torch.float32, device=x1.device)
+    need = lib.km_index_bwd_workspace_size(row_index.numel())
+    workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=x1.device)
+    bi_ptrs, bi_strides, _keep = _batch_index_args(batch_indices, rank)
+    with torch.cuda.device(x1.device):
+        status = lib.km_index_bwd(
+            kid, rank, _i64(batch_shape), x1.shape[-1], x2.shape[-1],
+            *_tensor_args(x1), *_tensor_args(x2), *_tensor_args(params),
+            *_tensor_args(start), *_tensor_args(end),
+            len(shape), _i64(shape), bi_ptrs, bi_strides,
+            *_tensor_args(row_index), *_tensor_args(col_index), *_tensor_args(out_grad),
+            _ptr(grad), ctypes.c_void_p(workspace.data_ptr()), need, _stream(x1.device),
+        )
+    if status != 0:
+        _raise(lib, status)
+    return grad
+
+
+def dense(kernel_type: str, x1: Tensor, x2: Tensor, params: Tensor, start: Tensor,
+          end: Tensor) -> Tensor:
+    """Masked kernel matrix [..., m, n]   (C ABI: km_dense)."""
+    kid = _kernel_id(kernel_type)
+    batch_shape = _check_matrix_inputs(kernel_type, x1, x2, params, start, end)
+    lib = load_library()
+    out = torch.empty((*batch_shape, x1.shape[-1], x2.shape[-1]), dtype=torch.float32, device=x1.device)
+    with torch.cuda.device(x1.device):
+        status = lib.km_dense(
+            kid, len(batch_shape), _i64(batch_shape), x1.shape[-1], x2.shape[-1],
+            *_tensor_args(x1), *_tensor_args(x2), *_tensor_args(params),
+            *_tensor_args(start), *_tensor_args(end), _ptr(out), _stream(x1.device),
+        )
+    if status != 0:
+        _raise(lib, status)
+    return out
+
+
+def dense_bwd(kernel_type: str, x1: Tensor, x2: Tensor, params: Tensor, start: Tensor, end: Tensor,
+              out_grad: Tensor) -> Tensor:
+    """grad[..., P] of sum(out_grad * dense(...)) w.r.t. params   (C ABI: km_dense_bwd)."""
+    kid = _kernel_id(kernel_type)
+    check_cuda(out_grad)
+    check_float(out_grad)
+    batch_shape = _check_matrix_inputs(kernel_type, x1, x2, params, start, end)
+    _check_batch("out_grad", out_grad, batch_shape, 2)
+    m, n = x1.shape[-1], x2.shape[-1]
+    if tuple(out_grad.shape[-2:]) != (m, n):
+        raise RuntimeError(f"out_grad has shape {tuple(out_grad.shape)}, expected (..., {m}, {n})")
+    lib = load_library()
+    sizes = _i64(batch_shape)
+    grad = torch.empty((*batch_shape, params.shape[-1]), dtype=torch.float32, device=x1.device)
+    need = lib.km_param_grad_workspace_size(kid, len(batch_shape), sizes, m, n, 0)
+    workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=x1.device)
+    with torch.cuda.device(x1.device):
+        status = lib.km_dense_bwd(
+            kid, len(batch_shape), sizes, m, n,
+            *_tensor_args(x1), *_tensor_args(x2), *_tensor_args(params),
+            *_tensor_args(start), *_tensor_args(end), *_tensor_args(out_grad),
+            _ptr(grad), ctypes.c_void_p(workspace.data_ptr()), need, _stream(x1.device),
+        )
+    if status != 0:
+        _raise(lib, status)
+    return grad
 
 
 # -- ranges ------------------------------------------------------------------------------

@@ -28,7 +28,8 @@ _KERNEL_DEFINES = {
     "KERNEL_LOCALLY_PERIODIC": "locally_periodic",
 }
 
-_OPERATORS = ("matmul", "matmul_bwd", "bilinear_derivative", "index")
+_OPERATORS = ("matmul", "matmul_bwd", "bilinear_derivative", "index", "index_bwd", "dense",
+              "dense_bwd")
 
 
 @contextmanager
@@ -134,11 +135,24 @@ class NativeModule:
             x1, x2, left_vecs, right_vecs, params, start, end = args
             self._check_batch_dim(x1)
             result = _native.param_grad(kt, x1, x2, left_vecs, right_vecs, params, start, end)
-        else:
+        elif self.op == "index":
             x1, x2, params, start, end, batch_indices, row_index, col_index = args
             self._check_batch_dim(x1)
             result = _native.index(kt, x1, x2, params, start, end, batch_indices, row_index,
                                    col_index)
+        elif self.op == "index_bwd":
+            x1, x2, params, start, end, batch_indices, row_index, col_index, out_grad = args
+            self._check_batch_dim(x1)
+            result = _native.index_bwd(kt, x1, x2, params, start, end, batch_indices, row_index,
+                                       col_index, out_grad)
+        elif self.op == "dense":
+            x1, x2, params, start, end = args
+            self._check_batch_dim(x1)
+            result = _native.dense(kt, x1, x2, params, start, end)
+        else:
+            x1, x2, params, start, end, out_grad = args
+            self._check_batch_dim(x1)
+            result = _native.dense_bwd(kt, x1, x2, params, start, end, out_grad)
         if self.debug:
             # Debug builds of the reference synchronise and check after every launch
             # (native/common/gpu_assert.cuh:6-23).

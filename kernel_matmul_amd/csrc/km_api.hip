@@ -491,4 +491,206 @@ int km_index(int kernel_type, int batch_rank, const int64_t* batch_sizes, int64_
     return err == hipSuccess ? KM_OK : fail_hip(op, err);
 }
 
+
+// ---------------------------------------------------------------------------------------
+// index_bwd
+// ---------------------------------------------------------------------------------------
+size_t km_index_bwd_workspace_size(int64_t num_entries) {
+    return num_entries > 0 ? index_bwd_workspace_bytes(num_entries) : 0;
+}
+
+int km_index_bwd(int kernel_type, int batch_rank, const int64_t* batch_sizes, int64_t m, int64_t n,
+                 const float* x1, const int64_t* x1_strides, const float* x2,
+                 const int64_t* x2_strides, const float* params, const int64_t* params_strides,
+                 const int32_t* start, const int64_t* start_strides, const int32_t* end,
+                 const int64_t* end_strides, int index_rank, const int64_t* index_sizes,
+                 const int32_t* const* batch_index, const int64_t* const* batch_index_strides,
+                 const int32_t* row_index, const int64_t* row_index_strides,
+                 const int32_t* col_index, const int64_t* col_index_strides,
+                 const float* out_grad, const int64_t* out_grad_strides, float* grad,
+                 void* workspace, size_t workspace_bytes, void* stream) {
+    const char* op = "km_index_bwd";
+    long long nb = 0;
+    if (int rc = check_common(op, kernel_type, batch_rank, batch_sizes, m, n, &nb)) return rc;
+    if (index_rank < 1 || index_rank > KM_MAX_BATCH_RANK + 1) {
+        return fail(KM_ERR_UNSUPPORTED, "%s: index rank %d outside [1, %d]", op, index_rank,
+                    KM_MAX_BATCH_RANK + 1);
+    }
+    KM_REQUIRE_PTR(op, index_sizes);
+    long long total = 1;
+    for (int d = 0; d < index_rank; d++) {
+        if (index_sizes[d] < 0) return fail(KM_ERR_INVALID_ARGUMENT, "%s: negative index size", op);
+        total *= index_sizes[d];
+        if (total > INT_LIMIT) return fail(KM_ERR_UNSUPPORTED, "%s: too many index entries", op);
+    }
+    if (nb == 0) return KM_OK;
+    KM_REQUIRE_PTR(op, grad);
+    KM_REQUIRE_PTR(op, params);
+    KM_REQUIRE_PTR(op, params_strides);
+    KM_REQUIRE_PTR(op, x1_strides);
+    KM_REQUIRE_PTR(op, x2_strides);
+    KM_REQUIRE_PTR(op, start_strides);
+    KM_REQUIRE_PTR(op, end_strides);
+    if (total > 0) {
+        KM_REQUIRE_PTR(op, row_index);
+        KM_REQUIRE_PTR(op, row_index_strides);
+        KM_REQUIRE_PTR(op, col_index);
+        KM_REQUIRE_PTR(op, col_index_strides);
+        KM_REQUIRE_PTR(op, out_grad);
+        KM_REQUIRE_PTR(op, out_grad_strides);
+        if (batch_rank > 0) {
+            KM_REQUIRE_PTR(op, batch_index);
+            KM_REQUIRE_PTR(op, batch_index_strides);
+            for (int d = 0; d < batch_rank; d++) {
+                if (batch_index[d] == nullptr || batch_index_strides[d] == nullptr) {
+                    return fail(KM_ERR_INVALID_ARGUMENT, "%s: batch_index[%d] is NULL", op, d);
+                }
+            }
+        }
+    }
+    const bool empty = m == 0 || n == 0;
+    if (!empty && total > 0) {
+        KM_REQUIRE_PTR(op, x1);
+        KM_REQUIRE_PTR(op, x2);
+        KM_REQUIRE_PTR(op, start);
+        KM_REQUIRE_PTR(op, end);
+    }
+    const size_t need = km_index_bwd_workspace_size(total);
+    if (need > 0 && (workspace == nullptr || workspace_bytes < need)) {
+        return fail(KM_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", op, need,
+                    workspace ? workspace_bytes : (size_t)0);
+    }
+    IndexBwdProblem p;
+    p.index.kernel_type = kernel_type;
+    p.index.batch_rank = batch_rank;
+    p.index.batch_sizes = batch_sizes;
+    p.index.m = empty ? 0 : m;
+    p.index.n = empty ? 0 : n;
+    p.index.x1 = x1;
+    p.index.x1_strides = x1_strides;
+    p.index.x2 = x2;
+    p.index.x2_strides = x2_strides;
+    p.index.params = params;
+    p.index.params_strides = params_strides;
+    p.index.start = start;
+    p.index.start_strides = start_strides;
+    p.index.end = end;
+    p.index.end_strides = end_strides;
+    p.index.index_rank = index_rank;
+    p.index.index_sizes = index_sizes;
+    p.index.batch_index = batch_index;
+    p.index.batch_index_strides = batch_index_strides;
+    p.index.row_index = row_index;
+    p.index.row_index_strides = row_index_strides;
+    p.index.col_index = col_index;
+    p.index.col_index_strides = col_index_strides;
+    p.index.out = nullptr;
+    p.num_batches = nb;
+    p.out_grad = out_grad;
+    p.out_grad_strides = out_grad_strides;
+    p.grad = grad;
+    p.workspace = workspace;
+    hipError_t err = launch_index_bwd(p, (hipStream_t)stream);
+    return err == hipSuccess ? KM_OK : fail_hip(op, err);
+}
+
+// ---------------------------------------------------------------------------------------
+// dense / dense_bwd
+// ---------------------------------------------------------------------------------------
+static int fill_dense(const char* op, DenseProblem* p, int kernel_type, int batch_rank,
+                      const int64_t* batch_sizes, int64_t m, int64_t n, const float* x1,
+                      const int64_t* x1_strides, const float* x2, const int64_t* x2_strides,
+                      const float* params, const int64_t* params_strides, const int32_t* start,
+                      const int64_t* start_strides, const int32_t* end, const int64_t* end_strides,
+                      long long* nb) {
+    if (int rc = check_common(op, kernel_type, batch_rank, batch_sizes, m, n, nb)) return rc;
+    if (*nb == 0) return KM_OK;
+    KM_REQUIRE_PTR(op, params);
+    KM_REQUIRE_PTR(op, params_strides);
+    KM_REQUIRE_PTR(op, x1_strides);
+    KM_REQUIRE_PTR(op, x2_strides);
+    KM_REQUIRE_PTR(op, start_strides);
+    KM_REQUIRE_PTR(op, end_strides);
+    if (m > 0) {
+        KM_REQUIRE_PTR(op, x1);
+        KM_REQUIRE_PTR(op, start);
+        KM_REQUIRE_PTR(op, end);
+    }
+    if (n > 0) KM_REQUIRE_PTR(op, x2);
+    p->kernel_type = kernel_type;
+    p->batch_rank = batch_rank;
+    p->batch_sizes = batch_sizes;
+    p->num_batches = *nb;
+    p->m = m;
+    p->n = n;
+    p->x1 = x1;
+    p->x1_strides = x1_strides;
+    p->x2 = x2;
+    p->x2_strides = x2_strides;
+    p->params = params;
+    p->params_strides = params_strides;
+    p->start = start;
+    p->start_strides = start_strides;
+    p->end = end;
+    p->end_strides = end_strides;
+    p->out = nullptr;
+    p->weights = nullptr;
+    p->weights_strides = nullptr;
+    p->grad = nullptr;
+    p->workspace = nullptr;
+    return KM_OK;
+}
+
+int km_dense(int kernel_type, int batch_rank, const int64_t* batch_sizes, int64_t m, int64_t n,
+             const float* x1, const int64_t* x1_strides, const float* x2,
+             const int64_t* x2_strides, const float* params, const int64_t* params_strides,
+             const int32_t* start, const int64_t* start_strides, const int32_t* end,
+             const int64_t* end_strides, float* out, void* stream) {
+    const char* op = "km_dense";
+    DenseProblem p;
+    long long nb = 0;
+    if (int rc = fill_dense(op, &p, kernel_type, batch_rank, batch_sizes, m, n, x1, x1_strides, x2,
+                            x2_strides, params, params_strides, start, start_strides, end,
+                            end_strides, &nb)) {
+        return rc;
+    }
+    if (nb == 0 || m == 0 || n == 0) return KM_OK;
+    KM_REQUIRE_PTR(op, out);
+    p.out = out;
+    hipError_t err = launch_dense(p, (hipStream_t)stream);
+    return err == hipSuccess ? KM_OK : fail_hip(op, err);
+}
+
+int km_dense_bwd(int kernel_type, int batch_rank, const int64_t* batch_sizes, int64_t m, int64_t n,
+                 const float* x1, const int64_t* x1_strides, const float* x2,
+                 const int64_t* x2_strides, const float* params, const int64_t* params_strides,
+                 const int32_t* start, const int64_t* start_strides, const int32_t* end,
+                 const int64_t* end_strides, const float* out_grad,
+                 const int64_t* out_grad_strides, float* grad, void* workspace,
+                 size_t workspace_bytes, void* stream) {
+    const char* op = "km_dense_bwd";
+    DenseProblem p;
+    long long nb = 0;
+    if (int rc = fill_dense(op, &p, kernel_type, batch_rank, batch_sizes, m, n, x1, x1_strides, x2,
+                            x2_strides, params, params_strides, start, start_strides, end,
+                            end_strides, &nb)) {
+        return rc;
+    }
+    if (nb == 0) return KM_OK;
+    KM_REQUIRE_PTR(op, grad);
+    KM_REQUIRE_PTR(op, out_grad_strides);
+    if (m > 0 && n > 0) KM_REQUIRE_PTR(op, out_grad);
+    const size_t need = km_param_grad_workspace_size(kernel_type, batch_rank, batch_sizes, m, n, 0);
+    if (need > 0 && (workspace == nullptr || workspace_bytes < need)) {
+        return fail(KM_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", op, need,
+                    workspace ? workspace_bytes : (size_t)0);
+    }
+    p.weights = out_grad;
+    p.weights_strides = out_grad_strides;
+    p.grad = grad;
+    p.workspace = workspace;
+    hipError_t err = launch_dense_bwd(p, (hipStream_t)stream);
+    return err == hipSuccess ? KM_OK : fail_hip(op, err);
+}
+
 }  // extern "C"

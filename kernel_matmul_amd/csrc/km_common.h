@@ -162,4 +162,74 @@ __device__ __forceinline__ float kernel_value(float x1, float x2, const KernelCo
     }
 }
 
+// Sum over the 64 lanes of a wavefront (every lane receives the total).
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        v += __shfl_xor(v, off, 64);
+    }
+    return v;
+}
+
+// Accumulates the per-pair derivative terms.  acc[] meaning per kernel type:
+//   rbf      : acc0 = sum C E u^2,  acc1 = sum C E
+//   spectral : acc0 = sum C E cos u^2,  acc1 = sum C E sin d,  acc2 = sum C E cos
+//   loc.per. : acc0 = sum C E u^2,  acc1 = sum C E sin^2,  acc2 = sum C E sin cos d,  acc3 = sum C E
+// with E the kernel value without sigma.
+template <int KT>
+__device__ __forceinline__ void accumulate_pair(float x1, float x2, float coeff,
+                                                const KernelConsts& kc, float (&acc)[KM_MAX_PARAMS]) {
+    const float d = x1 - x2;
+    const float u = d * kc.s;
+    const float uu = u * u;
+    if (KT == KM_KERNEL_RBF) {
+        const float w = coeff * __builtin_amdgcn_exp2f(-uu);
+        acc[0] = __builtin_fmaf(w, uu, acc[0]);
+        acc[1] += w;
+    } else if (KT == KM_KERNEL_SPECTRAL) {
+        const float ph = d * kc.f;
+        const float w = coeff * __builtin_amdgcn_exp2f(-uu);
+        const float wc = w * __builtin_amdgcn_cosf(ph);
+        const float ws = w * __builtin_amdgcn_sinf(ph);
+        acc[0] = __builtin_fmaf(wc, uu, acc[0]);
+        acc[1] = __builtin_fmaf(ws, d, acc[1]);
+        acc[2] += wc;
+    } else {
+        const float ph = d * kc.f;
+        const float sn = __builtin_amdgcn_sinf(ph);
+        const float cs = __builtin_amdgcn_cosf(ph);
+        const float q = sn * sn;
+        const float w = coeff * __builtin_amdgcn_exp2f(__builtin_fmaf(-kc.cl, q, -uu));
+        acc[0] = __builtin_fmaf(w, uu, acc[0]);
+        acc[1] = __builtin_fmaf(w, q, acc[1]);
+        acc[2] = __builtin_fmaf(w * (sn * cs), d, acc[2]);
+        acc[3] += w;
+    }
+}
+
+// Chain rule from the accumulated sums of accumulate_pair back to the user parameters
+// (reference: native/common/kernel_function.cuh:221-251), written to g[0..P).
+template <int KT>
+__device__ __forceinline__ void finish_param_grad(double s0, double s1, double s2, double s3,
+                                                  const float* __restrict__ params,
+                                                  long long stride, float* __restrict__ g) {
+    const double l = (double)params[0];
+    const double sigma = (double)params[KernelTraits<KT>::SIGMA * stride];
+    if (KT == KM_KERNEL_RBF) {
+        g[0] = (float)(sigma * s0 * KM_2LN2 / l);
+        g[1] = (float)s1;
+    } else if (KT == KM_KERNEL_SPECTRAL) {
+        g[0] = (float)(sigma * s0 * KM_2LN2 / l);
+        g[1] = (float)(-2.0 * KM_PI * sigma * s1);
+        g[2] = (float)s2;
+    } else {
+        const double lp = (double)params[stride];
+        const double period = (double)params[2 * stride];
+        g[0] = (float)(sigma * s0 * KM_2LN2 / l);
+        g[1] = (float)(2.0 * sigma * s1 / (lp * lp));
+        g[2] = (float)(4.0 * KM_PI * sigma * s2 / (lp * period * period));
+        g[3] = (float)s3;
+    }
+}
+
 }  // namespace km

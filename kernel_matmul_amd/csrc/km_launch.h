@@ -96,6 +96,52 @@ struct IndexProblem {
 
 hipError_t launch_index(const IndexProblem& p, hipStream_t stream);
 
+// index_bwd: the index problem plus the incoming gradient (same shape as the index tensors),
+// the output [batch..., P] and scratch of index_bwd_workspace_bytes().
+struct IndexBwdProblem {
+    IndexProblem index;
+    long long num_batches;
+    const float* out_grad;
+    const int64_t* out_grad_strides;
+    float* grad;
+    void* workspace;
+};
+size_t index_bwd_workspace_bytes(long long total_entries);
+hipError_t launch_index_bwd(const IndexBwdProblem& p, hipStream_t stream);
+
+struct DenseProblem {
+    int kernel_type;
+    int batch_rank;
+    const int64_t* batch_sizes;
+    long long num_batches;
+    int64_t m, n;
+    const float* x1;
+    const int64_t* x1_strides;
+    const float* x2;
+    const int64_t* x2_strides;
+    const float* params;
+    const int64_t* params_strides;
+    const int32_t* start;
+    const int64_t* start_strides;
+    const int32_t* end;
+    const int64_t* end_strides;
+    float* out;                      // dense
+    const float* weights;            // dense_bwd: out_grad [batch..., m, n]
+    const int64_t* weights_strides;
+    float* grad;                     // dense_bwd: [batch..., P]
+    void* workspace;                 // dense_bwd
+};
+
+hipError_t launch_dense(const DenseProblem& p, hipStream_t stream);
+hipError_t launch_dense_bwd(const DenseProblem& p, hipStream_t stream);
+
+struct BatchShape;
+struct BatchStrides;
+hipError_t launch_param_grad_reduce(int kernel_type, const BatchShape& batch, long long num_batches,
+                                    long long partial_rows, const float* partials,
+                                    const float* params, const BatchStrides& params_bs,
+                                    long long params_s, float* grad, hipStream_t stream);
+
 hipError_t launch_make_ranges(const float* x1, const float* x2, int64_t num_batch, int64_t n1,
                               int64_t n2, float cutoff, int block_size, int align, int32_t* start,
                               int32_t* end, hipStream_t stream);

@@ -37,50 +37,6 @@ struct GradArgs {
     long long x1_s, x2_s, left_s0, left_s1, right_s0, right_s1, params_s, start_s, end_s;
 };
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) {
-        v += __shfl_xor(v, off, 64);
-    }
-    return v;
-}
-
-// Accumulates the per-pair derivative terms.  acc[] meaning per kernel type:
-//   rbf      : acc0 = sum C E u^2,  acc1 = sum C E
-//   spectral : acc0 = sum C E cos u^2,  acc1 = sum C E sin d,  acc2 = sum C E cos
-//   loc.per. : acc0 = sum C E u^2,  acc1 = sum C E sin^2,  acc2 = sum C E sin cos d,  acc3 = sum C E
-// with E the kernel value without sigma.
-template <int KT>
-__device__ __forceinline__ void accumulate_pair(float x1, float x2, float coeff,
-                                                const KernelConsts& kc, float (&acc)[KM_MAX_PARAMS]) {
-    const float d = x1 - x2;
-    const float u = d * kc.s;
-    const float uu = u * u;
-    if (KT == KM_KERNEL_RBF) {
-        const float w = coeff * __builtin_amdgcn_exp2f(-uu);
-        acc[0] = __builtin_fmaf(w, uu, acc[0]);
-        acc[1] += w;
-    } else if (KT == KM_KERNEL_SPECTRAL) {
-        const float ph = d * kc.f;
-        const float w = coeff * __builtin_amdgcn_exp2f(-uu);
-        const float wc = w * __builtin_amdgcn_cosf(ph);
-        const float ws = w * __builtin_amdgcn_sinf(ph);
-        acc[0] = __builtin_fmaf(wc, uu, acc[0]);
-        acc[1] = __builtin_fmaf(ws, d, acc[1]);
-        acc[2] += wc;
-    } else {
-        const float ph = d * kc.f;
-        const float sn = __builtin_amdgcn_sinf(ph);
-        const float cs = __builtin_amdgcn_cosf(ph);
-        const float q = sn * sn;
-        const float w = coeff * __builtin_amdgcn_exp2f(__builtin_fmaf(-kc.cl, q, -uu));
-        acc[0] = __builtin_fmaf(w, uu, acc[0]);
-        acc[1] = __builtin_fmaf(w, q, acc[1]);
-        acc[2] = __builtin_fmaf(w * (sn * cs), d, acc[2]);
-        acc[3] += w;
-    }
-}
-
 // TL > 0: the vector width c is at most 4*TL and the left operand stays in registers.
 // TL == 0: any c; the left operand is re-read (from L1/L2) for every column chunk.
 template <int KT, int TL>
@@ -257,24 +213,7 @@ __global__ void __launch_bounds__(256) param_grad_reduce(const ReduceArgs a) {
     batch_multi_index(a.batch, b, bidx);
     const float* __restrict__ params = a.params + batch_offset(a.batch, a.params_bs, bidx);
     float* __restrict__ g = a.grad + b * P;
-    const double s0 = sh[0][0], s1 = sh[1][0], s2 = sh[2][0], s3 = sh[3][0];
-    const double l = (double)params[0];
-    const double sigma = (double)params[KernelTraits<KT>::SIGMA * a.params_s];
-    if (KT == KM_KERNEL_RBF) {
-        g[0] = (float)(sigma * s0 * KM_2LN2 / l);
-        g[1] = (float)s1;
-    } else if (KT == KM_KERNEL_SPECTRAL) {
-        g[0] = (float)(sigma * s0 * KM_2LN2 / l);
-        g[1] = (float)(-2.0 * KM_PI * sigma * s1);
-        g[2] = (float)s2;
-    } else {
-        const double lp = (double)params[a.params_s];
-        const double period = (double)params[2 * a.params_s];
-        g[0] = (float)(sigma * s0 * KM_2LN2 / l);
-        g[1] = (float)(2.0 * sigma * s1 / (lp * lp));
-        g[2] = (float)(4.0 * KM_PI * sigma * s2 / (lp * period * period));
-        g[3] = (float)s3;
-    }
+    finish_param_grad<KT>(sh[0][0], sh[1][0], sh[2][0], sh[3][0], params, a.params_s, g);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -309,6 +248,33 @@ static hipError_t launch_partial(const GradArgs& a, unsigned grid_x, hipStream_t
         hipLaunchKernelGGL((param_grad_partial<KT, 4>), dim3(grid_x), dim3(64), 0, stream, a);
     } else {
         hipLaunchKernelGGL((param_grad_partial<KT, 0>), dim3(grid_x), dim3(64), 0, stream, a);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_param_grad_reduce(int kernel_type, const BatchShape& batch, long long num_batches,
+                                    long long partial_rows, const float* partials,
+                                    const float* params, const BatchStrides& params_bs,
+                                    long long params_s, float* grad, hipStream_t stream) {
+    ReduceArgs ra;
+    ra.batch = batch;
+    ra.partial_rows = partial_rows;
+    ra.partials = partials;
+    ra.params = params;
+    ra.params_bs = params_bs;
+    ra.params_s = params_s;
+    ra.grad = grad;
+    const unsigned rgrid = (unsigned)num_batches;
+    switch (kernel_type) {
+        case KM_KERNEL_RBF:
+            hipLaunchKernelGGL((param_grad_reduce<KM_KERNEL_RBF>), dim3(rgrid), dim3(256), 0, stream, ra);
+            break;
+        case KM_KERNEL_SPECTRAL:
+            hipLaunchKernelGGL((param_grad_reduce<KM_KERNEL_SPECTRAL>), dim3(rgrid), dim3(256), 0, stream, ra);
+            break;
+        default:
+            hipLaunchKernelGGL((param_grad_reduce<KM_KERNEL_LOCALLY_PERIODIC>), dim3(rgrid), dim3(256), 0, stream, ra);
+            break;
     }
     return hipGetLastError();
 }
@@ -360,27 +326,8 @@ hipError_t launch_param_grad(const ParamGradProblem& p, hipStream_t stream) {
         }
     }
 
-    ReduceArgs ra;
-    ra.batch = a.batch;
-    ra.partial_rows = row_blocks * a.col_splits;
-    ra.partials = a.partials;
-    ra.params = p.params;
-    ra.params_bs = a.params_bs;
-    ra.params_s = a.params_s;
-    ra.grad = p.grad;
-    const unsigned rgrid = (unsigned)p.num_batches;
-    switch (p.kernel_type) {
-        case KM_KERNEL_RBF:
-            hipLaunchKernelGGL((param_grad_reduce<KM_KERNEL_RBF>), dim3(rgrid), dim3(256), 0, stream, ra);
-            break;
-        case KM_KERNEL_SPECTRAL:
-            hipLaunchKernelGGL((param_grad_reduce<KM_KERNEL_SPECTRAL>), dim3(rgrid), dim3(256), 0, stream, ra);
-            break;
-        default:
-            hipLaunchKernelGGL((param_grad_reduce<KM_KERNEL_LOCALLY_PERIODIC>), dim3(rgrid), dim3(256), 0, stream, ra);
-            break;
-    }
-    return hipGetLastError();
+    return launch_param_grad_reduce(p.kernel_type, a.batch, p.num_batches, row_blocks * a.col_splits,
+                                    a.partials, p.params, a.params_bs, a.params_s, p.grad, stream);
 }
 
 }  // namespace km

@@ -26,6 +26,9 @@ from torch import Size, Tensor, dtype
 from kernel_matmul_amd import _BLOCK_SIZE, ranges
 from kernel_matmul_amd.configurations import (
     BilinearDerivativeConfiguration,
+    DenseBwdConfiguration,
+    DenseConfiguration,
+    IndexBwdConfiguration,
     IndexConfiguration,
     MatmulAutotuneConfiguration,
     MatmulBwdConfiguration,
@@ -153,6 +156,20 @@ class _MatmulOperator(torch.autograd.Function):
         return None, None, grad_rhs, grad_params, None, None, None, None, None
 
 
+class _DenseOperator(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x1, x2, params, start, end, native_dense, native_dense_bwd):
+        ctx.save_for_backward(x1, x2, params, start, end)
+        ctx.native_dense_bwd = native_dense_bwd
+        return native_dense(x1, x2, params, start, end)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        x1, x2, params, start, end = ctx.saved_tensors
+        grad = ctx.native_dense_bwd(x1, x2, params, start, end, grad_output)
+        return None, None, grad, None, None, None, None
+
+
 class _IndexOperator(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x1, x2, params, start, end, native_index, native_index_bwd, row_index,
@@ -165,8 +182,6 @@ class _IndexOperator(torch.autograd.Function):
     def backward(ctx, grad_output):
         x1, x2, params, start, end, row_index, col_index = ctx.saved_tensors[:7]
         batch_indices = ctx.saved_tensors[7:]
-        if ctx.native_index_bwd is None:
-            raise NotImplementedError("gradients through indexed entries are not available yet")
         grad = ctx.native_index_bwd(
             x1, x2, params, start, end, batch_indices, row_index, col_index, grad_output
         )
@@ -228,7 +243,9 @@ class KernelMatmulLinearOperator(LinearOperator):
             "bilinear_derivative", BilinearDerivativeConfiguration(kernel_type)
         )
         self._native_index = NativeFunction("index", IndexConfiguration(kernel_type))
-        self._native_index_bwd = None
+        self._native_index_bwd = NativeFunction("index_bwd", IndexBwdConfiguration(kernel_type))
+        self._native_dense = NativeFunction("dense", DenseConfiguration(kernel_type))
+        self._native_dense_bwd = NativeFunction("dense_bwd", DenseBwdConfiguration(kernel_type))
 
     # -- helpers -------------------------------------------------------------------------
     def _get_args_for_native(self, batch_shape) -> tuple[Tensor, Tensor, Tensor, Tensor, Tensor]:
@@ -270,16 +287,10 @@ class KernelMatmulLinearOperator(LinearOperator):
         )
 
     def to_dense(self) -> Tensor:
-        """Materialise the masked matrix (through the index operator, entry by entry)."""
-        m, n = self._x1.size(-2), self._x2.size(-2)
-        device = self._x1.device
-        grids = torch.meshgrid(
-            *(torch.arange(s, device=device) for s in self._batch_shape),
-            torch.arange(m, device=device),
-            torch.arange(n, device=device),
-            indexing="ij",
+        x1, x2, params, start, end = self._get_args_for_native(self._batch_shape)
+        return _DenseOperator.apply(
+            x1, x2, params, start, end, self._native_dense, self._native_dense_bwd
         )
-        return self._get_indices(grids[-2], grids[-1], *grids[:-2])
 
     def _expand_batch(self, batch_shape: Size | List[int]) -> "KernelMatmulLinearOperator":
         return KernelMatmulLinearOperator(

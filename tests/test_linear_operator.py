@@ -142,3 +142,27 @@ def test_rhs_gradient_needs_aligned_pattern():
     rhs = torch.randn(280, 2, device=device, requires_grad=True)
     with pytest.raises(RuntimeError, match="align=True"):
         op._matmul(rhs).sum().backward()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kernel_type", ["rbf", "spectral", "locally_periodic"])
+def test_autograd_through_to_dense_and_diagonal(kernel_type):
+    device = torch.device("cuda:0")
+    batch = (2,)
+    op, params, a = _make_operator(kernel_type, batch, 300, 300, device, True, requires_grad=True)
+    weight = torch.randn(2, 300, 300, device=device)
+    (op.to_dense() * weight).sum().backward()
+    bc = lambda v: np.broadcast_to(v, (*batch, *v.shape))
+    grads = oracle.kernel_matrix_grad(kernel_type, bc(a["x1"]), bc(a["x2"]), a["params"])
+    mask = oracle.range_mask(bc(a["start"]), bc(a["end"]), 300, 300)
+    expected = np.sum(np.where(mask, weight.cpu().double().numpy(), 0.0)[..., None, :, :] * grads, axis=(-2, -1))
+    scale = np.abs(expected).max(axis=-1, keepdims=True)
+    assert np.all(np.abs(params.grad.cpu().numpy() - expected) <= 1e-5 + 1e-4 * scale)
+
+    params.grad = None
+    dweight = torch.randn(2, 300, device=device)
+    (op.diagonal() * dweight).sum().backward()
+    diag_grads = np.diagonal(grads, axis1=-2, axis2=-1)  # [b, P, n]
+    expected = np.sum(diag_grads * dweight.cpu().double().numpy()[:, None, :], axis=-1)
+    scale = np.abs(expected).max(axis=-1, keepdims=True)
+    assert np.all(np.abs(params.grad.cpu().numpy() - expected) <= 1e-5 + 1e-4 * scale)

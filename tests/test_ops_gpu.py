@@ -120,3 +120,64 @@ def test_index(example_data, shape):
     assert_close(result, expected)
     # entries outside the pattern are exactly zero
     assert torch.all(result[torch.from_numpy(expected == 0.0).to(device)] == 0.0)
+
+
+def test_dense(example_data):
+    d = example_data
+    args = (d.x1, d.x2, d.params, d.start, d.end)
+    from kernel_matmul_amd.configurations import DenseConfiguration
+
+    result = load_native("dense", DenseConfiguration(d.kernel_type).make_config(args)).call(*args)
+    a = d.numpy()
+    expected = oracle.dense(d.kernel_type, a["x1"], a["x2"], a["params"], a["start"], a["end"])
+    assert_close(result, expected)
+    assert torch.all(result[torch.from_numpy(expected == 0.0).to(result.device)] == 0.0)
+
+
+def test_dense_bwd(example_data):
+    d = example_data
+    from kernel_matmul_amd.configurations import DenseBwdConfiguration
+
+    out_grad = torch.randn(*d.params.shape[:-1], d.x1.shape[-1], d.x2.shape[-1])
+    out_grad = (out_grad / torch.linalg.norm(out_grad, dim=(-2, -1), keepdim=True)).to(d.x1.device)
+    args = (d.x1, d.x2, d.params, d.start, d.end, out_grad)
+    result = load_native("dense_bwd", DenseBwdConfiguration(d.kernel_type).make_config(args)).call(*args)
+    a = d.numpy()
+    grads = oracle.kernel_matrix_grad(d.kernel_type, a["x1"], a["x2"], a["params"])
+    mask = oracle.range_mask(a["start"], a["end"], grads.shape[-2], grads.shape[-1])
+    weights = np.where(mask, out_grad.cpu().double().numpy(), 0.0)
+    expected = np.sum(weights[..., None, :, :] * grads, axis=(-2, -1))
+    err = np.abs(result.cpu().double().numpy() - expected)
+    assert np.all(err <= _grad_tolerance(expected)), (result.cpu().numpy(), expected)
+
+
+@pytest.mark.square
+@pytest.mark.parametrize("shape", [(100,), (5, 101)])
+def test_index_bwd(example_data, shape):
+    d = example_data
+    from kernel_matmul_amd.configurations import IndexBwdConfiguration
+
+    device = d.x1.device
+    m, n = d.x1.shape[-1], d.x2.shape[-1]
+    batch_indices = tuple(
+        torch.randint(0, size, shape, dtype=torch.int32).to(device) for size in d.params.shape[:-1]
+    )
+    row_index = torch.randint(0, m, shape, dtype=torch.int32).to(device)
+    col_index = torch.clamp(row_index + torch.randint(-40, 40, shape, dtype=torch.int32).to(device), 0, n - 1)
+    out_grad = torch.randn(shape).to(device)
+    args = (d.x1, d.x2, d.params, d.start, d.end, batch_indices, row_index, col_index, out_grad)
+    result = load_native("index_bwd", IndexBwdConfiguration(d.kernel_type).make_config(args)).call(*args)
+    a = d.numpy()
+    grads = oracle.kernel_matrix_grad(d.kernel_type, a["x1"], a["x2"], a["params"])  # [..., P, m, n]
+    mask = oracle.range_mask(a["start"], a["end"], m, n)
+    bi = [b.cpu().numpy().astype(np.int64).ravel() for b in batch_indices]
+    rows = row_index.cpu().numpy().astype(np.int64).ravel()
+    cols = col_index.cpu().numpy().astype(np.int64).ravel()
+    og = out_grad.cpu().double().numpy().ravel()
+    expected = np.zeros(a["params"].shape, dtype=np.float64)
+    for q in range(rows.size):
+        b = tuple(x[q] for x in bi)
+        if mask[b + (rows[q], cols[q])]:
+            expected[b] += og[q] * grads[b + (slice(None), rows[q], cols[q])]
+    err = np.abs(result.cpu().double().numpy() - expected)
+    assert np.all(err <= _grad_tolerance(expected) + 1e-6), (result.cpu().numpy(), expected)
