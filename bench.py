@@ -79,7 +79,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="headline", choices=sorted(WORKLOADS))
-    ap.add_argument("--variant", default="auto", choices=["auto", "mfma_f32", "mfma_f16", "valu"])
+    ap.add_argument("--variant", default="auto", choices=["auto", "mfma_f32", "mfma_f16", "mfma_f16_direct", "valu"])
     ap.add_argument("--rows-per-wave", type=int, default=0)
     ap.add_argument("--col-splits", type=int, default=0)
     ap.add_argument("--batch", type=int, default=None, help="override the number of batch items")
@@ -205,7 +205,7 @@ def main() -> int:
         },
         "roofline": {
             "bound": "mfma",
-            "kernel": "km::param_grad_partial" if is_grad else {"auto": "km::fwd_mfma_f16", "mfma_f16": "km::fwd_mfma_f16", "mfma_f32": "km::fwd_mfma_f32", "valu": "km::fwd_valu"}[args.variant],
+            "kernel": "km::param_grad_partial" if is_grad else {"auto": "km::fwd_spectral_f16", "mfma_f16": "km::fwd_spectral_f16", "mfma_f16_direct": "km::fwd_mfma_f16", "mfma_f32": "km::fwd_mfma_f32", "valu": "km::fwd_valu"}[args.variant],
             "achieved": achieved_tflops,
             "peak": PEAK_FP32_TFLOPS,
             "unit": "TFLOP/s",

@@ -53,7 +53,9 @@ extern "C" {
  * only select among ahead-of-time instantiated kernels. */
 typedef struct km_launch_options {
     int variant;          /* 0 = table, 1 = VALU FMA contraction, 2 = fp32 MFMA contraction,
-                             3 = split-fp16 (hi+lo) MFMA contraction with fp32 accumulation */
+                             3 = split-fp16 (hi+lo) MFMA contraction with fp32 accumulation
+                             (spectral kernels in phase-split form), 4 = the same with the
+                             cosine evaluated per pair */
     int rows_per_wave;    /* 0 = table; else 16, 32, 64 or 128 rows of x1 per wavefront */
     int col_splits;       /* 0 = table; else 1, 2, 4 or 8 wavefronts sharing one row range */
     int reserved;

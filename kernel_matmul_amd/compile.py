@@ -106,7 +106,7 @@ class NativeModule:
             options.col_splits = max(s for s in (1, 2, 4, 8) if s <= col_blocks)
         variant = self.defines.get("MATMUL_VARIANT")
         if variant is not None:
-            options.variant = {"auto": 0, "valu": 1, "mfma": 2, "mfma_f32": 2, "mfma_f16": 3}[variant]
+            options.variant = {"auto": 0, "valu": 1, "mfma": 2, "mfma_f32": 2, "mfma_f16": 3, "mfma_f16_direct": 4}[variant]
         rows = self.defines.get("MATMUL_ROWS_PER_WAVE")
         if rows is not None:
             options.rows_per_wave = int(rows)

@@ -86,7 +86,8 @@ static int make_plan(const MatmulProblem& p, const km_launch_options* opt, Matmu
     if (variant == KM_VARIANT_AUTO) {
         variant = KM_VARIANT_MFMA_F16;
     }
-    if (variant != KM_VARIANT_VALU && variant != KM_VARIANT_MFMA_F32 && variant != KM_VARIANT_MFMA_F16) {
+    if (variant != KM_VARIANT_VALU && variant != KM_VARIANT_MFMA_F32 && variant != KM_VARIANT_MFMA_F16 &&
+        variant != KM_VARIANT_MFMA_F16_DIRECT) {
         return fail(KM_ERR_INVALID_ARGUMENT, "km_matmul: unknown variant %d", variant);
     }
     plan->variant = variant;
@@ -94,9 +95,18 @@ static int make_plan(const MatmulProblem& p, const km_launch_options* opt, Matmu
         plan->k_chunk = p.k > 8 ? 16 : (p.k > 4 ? 8 : 4);
         plan->row_groups = 8;
         plan->col_splits = 1;
+        plan->tail_balance = 0;
         return KM_OK;
     }
-    plan->k_chunk = p.k <= 16 ? 16 : (p.k <= 32 ? 32 : 64);
+    // The phase-split spectral kernel keeps two accumulator sets per rhs column group, so it
+    // takes at most 32 rhs columns per pass.
+    const bool phase_split = variant == KM_VARIANT_MFMA_F16 && p.kernel_type == KM_KERNEL_SPECTRAL && p.k <= 16;
+    if (variant == KM_VARIANT_MFMA_F16 && !phase_split) {
+        // Only spectral kernels with up to 16 rhs columns gain from the phase-split form.
+        variant = KM_VARIANT_MFMA_F16_DIRECT;
+        plan->variant = variant;
+    }
+    plan->k_chunk = p.k <= 16 ? 16 : ((p.k <= 32 || phase_split) ? 32 : 64);
     const int G = plan->k_chunk / 16;
     const long long row_blocks = (p.m + KM_BLOCK_SIZE - 1) / KM_BLOCK_SIZE;
     const long long base = row_blocks * p.num_batches * ((p.k + plan->k_chunk - 1) / plan->k_chunk);
@@ -126,18 +136,21 @@ static int make_plan(const MatmulProblem& p, const km_launch_options* opt, Matmu
     }
     // Register budget of the split-fp16 kernel: its operand buffers grow with G, so wide rhs
     // tiles get fewer row groups per wavefront (no spills, at least two wavefronts per SIMD).
-    if (variant == KM_VARIANT_MFMA_F16) {
-        const int max_r = G == 1 ? 8 : (G == 2 ? 4 : 2);
+    if (variant == KM_VARIANT_MFMA_F16 || variant == KM_VARIANT_MFMA_F16_DIRECT) {
+        const int groups = phase_split ? 2 * G : G;
+        const int max_r = groups == 1 ? 8 : (groups == 2 ? (phase_split ? 8 : 4) : (groups == 4 ? (phase_split ? 4 : 2) : 2));
         if (R > max_r) {
             R = max_r;
         }
     }
-    // The cross-wavefront reduction buffer (S * R * G KiB) must fit 64 KiB of LDS.
-    while (S > 1 && S * R * G > 64) {
+    // LDS per workgroup must stay within 64 KiB: the cross-wavefront reduction buffer takes
+    // S * R * G KiB and the phase-split kernel's tables 6 KiB per wavefront.
+    while (S > 1 && S * (R * G + (phase_split ? 6 : 0)) > 64) {
         S /= 2;
     }
     plan->row_groups = R;
     plan->col_splits = S;
+    plan->tail_balance = !(opt && opt->reserved == 1);  // reserved = 1 switches it off (measurements)
     return KM_OK;
 }
 

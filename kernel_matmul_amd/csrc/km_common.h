@@ -101,6 +101,7 @@ struct KernelConsts {
     float lsig;  // log2 |sigma|
     float cl;    // locally periodic: 2 log2(e) / lengthscale_periodic
     float sgn;   // sign of sigma (+1 / -1)
+    float one;   // 1.0 that is only known at run time (keeps x * one + y an fma)
 };
 
 template <int KT>
@@ -140,6 +141,7 @@ __device__ __forceinline__ KernelConsts make_consts(const float* __restrict__ pa
     const float sigma = params[KernelTraits<KT>::SIGMA * stride];
     c.sgn = sigma < 0.0f ? -1.0f : 1.0f;
     c.lsig = fold_sigma ? log2f(fabsf(sigma)) : 0.0f;
+    c.one = stride >= 0 ? 1.0f : 0.0f;  // strides are never negative
     return c;
 }
 

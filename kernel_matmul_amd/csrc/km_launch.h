@@ -7,7 +7,13 @@
 
 namespace km {
 
-enum { KM_VARIANT_AUTO = 0, KM_VARIANT_VALU = 1, KM_VARIANT_MFMA_F32 = 2, KM_VARIANT_MFMA_F16 = 3 };
+enum {
+    KM_VARIANT_AUTO = 0,
+    KM_VARIANT_VALU = 1,
+    KM_VARIANT_MFMA_F32 = 2,
+    KM_VARIANT_MFMA_F16 = 3,         // split-fp16 MFMA; spectral kernels in phase-split form
+    KM_VARIANT_MFMA_F16_DIRECT = 4   // split-fp16 MFMA with the cosine evaluated per pair
+};
 
 struct MatmulProblem {
     int kernel_type;
@@ -36,6 +42,7 @@ struct MatmulPlan {
     int k_chunk;     // rhs columns handled per workgroup (MFMA: 16/32/64, VALU: 4/8/16)
     int row_groups;  // MFMA: groups of 16 rows per wavefront (1, 2, 4, 8)
     int col_splits;  // MFMA: wavefronts per workgroup sharing one column range (1, 2, 4, 8)
+    int tail_balance;  // split-fp16 kernels: cut the uneven remainder into 16-row pieces
 };
 
 hipError_t launch_matmul(const MatmulProblem& p, const MatmulPlan& plan, hipStream_t stream);

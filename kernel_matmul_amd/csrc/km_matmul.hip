@@ -26,6 +26,26 @@ typedef _Float16 half8v __attribute__((ext_vector_type(8)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float float2v __attribute__((ext_vector_type(2)));
 
+#ifdef KM_TIMELINE
+// Development aid (never defined in the library build): per-wavefront placement and
+// start/end timestamps for timeline analysis.
+__device__ unsigned long long* g_timeline;
+#define KM_TL_BEGIN() const unsigned long long tl_begin = wall_clock64()
+#define KM_TL_END()                                                                          \
+    do {                                                                                     \
+        if ((threadIdx.x & 63) == 0) {                                                       \
+            const long long tl_id = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6); \
+            g_timeline[tl_id * 4 + 0] = __builtin_amdgcn_s_getreg((31 << 11) | 4);           \
+            g_timeline[tl_id * 4 + 1] = __builtin_amdgcn_s_getreg((3 << 11) | 20);           \
+            g_timeline[tl_id * 4 + 2] = tl_begin;                                            \
+            g_timeline[tl_id * 4 + 3] = wall_clock64();                                      \
+        }                                                                                    \
+    } while (0)
+#else
+#define KM_TL_BEGIN()
+#define KM_TL_END()
+#endif
+
 struct FwdArgs {
     BatchShape batch;
     long long num_batches;
@@ -33,6 +53,7 @@ struct FwdArgs {
     long long items_per_xcd;
     int m, n, k;
     int chunks_per_block;    // 128 / rows per workgroup
+    int tail_items;          // per XCD: row-block items at the end that are split 8 ways by rows
     const float* x1;
     const float* x2;
     const float* rhs;
@@ -74,6 +95,42 @@ __device__ __forceinline__ WaveView wave_view(const FwdArgs& a, long long item, 
     w.range_start = max(a.start[batch_offset(a.batch, a.start_bs, bidx) + w.row_block * a.start_s], 0);
     w.range_end = min(a.end[batch_offset(a.batch, a.end_bs, bidx) + w.row_block * a.end_s], a.n);
     return w;
+}
+
+
+// Work item of this workgroup.  Items are (row chunk, batch item) pairs, contiguous ranges of
+// which belong to one XCD (see xcd_item).  When the launch has a "tail" (only with 128 rows per
+// wavefront), the last `tail_items` items of every XCD are cut into 8 pieces of 16 rows that are
+// dispatched last: wavefronts are handed out in order, so these short pieces fill the SIMDs
+// that would otherwise idle while others finish a last full-size wavefront.
+struct ItemRef {
+    bool valid;
+    bool small;        // a 16-row piece of a tail item
+    long long item;    // (row chunk, batch) index
+    int piece;         // which 16-row piece (small only)
+};
+
+__device__ __forceinline__ ItemRef decode_item(const FwdArgs& a) {
+    ItemRef it;
+    it.small = false;
+    it.piece = 0;
+    if (a.tail_items == 0) {
+        it.item = xcd_item(blockIdx.x, a.items_per_xcd);
+    } else {
+        const unsigned xcd = blockIdx.x % KM_NUM_XCD;
+        const long long slot = blockIdx.x / KM_NUM_XCD;
+        const long long big = a.items_per_xcd - a.tail_items;
+        if (slot < big) {
+            it.item = (long long)xcd * a.items_per_xcd + slot;
+        } else {
+            const long long t = slot - big;
+            it.small = true;
+            it.item = (long long)xcd * a.items_per_xcd + big + t / 8;
+            it.piece = (int)(t % 8);
+        }
+    }
+    it.valid = it.item < a.total_items;
+    return it;
 }
 
 // Fixed-order reduction of the S wavefronts' accumulators through LDS and the masked store.
@@ -304,7 +361,7 @@ __global__ void __launch_bounds__(512) fwd_mfma_f32(const FwdArgs a) {
 
 template <int KT>
 __device__ __forceinline__ void kernel_pair_f16(float x1, float x2a, float x2b, const KernelConsts& c,
-                                                half2v* hi, half2v* lo) {
+                                                float one, half2v* hi, half2v* lo) {
     // Two neighbouring columns at once so that the conversions pack.
     float2v kv, res;
     float ea[2], ca[2];
@@ -332,19 +389,20 @@ __device__ __forceinline__ void kernel_pair_f16(float x1, float x2a, float x2b, 
 #pragma unroll
     for (int t = 0; t < 2; t++) {
         // Residual of the exact product where there is one (contracts to one fused op).
-        res[t] = KT == KM_KERNEL_SPECTRAL ? __builtin_fmaf(ea[t], ca[t], -(float)h[t])
-                                          : ea[t] - (float)h[t];
+        // Written as fma so that it maps to one v_fma_mix_f32 (fp16 operand read directly);
+        // `one` is a run-time 1.0 the compiler cannot fold away.
+        res[t] = __builtin_fmaf(ea[t], KT == KM_KERNEL_SPECTRAL ? ca[t] : one, -(float)h[t]);
     }
     *hi = h;
     *lo = __builtin_convertvector(res, half2v);
 }
 
-__device__ __forceinline__ void split_f16x8(const float (&v)[8], half8v* hi, half8v* lo) {
+__device__ __forceinline__ void split_f16x8(const float (&v)[8], float one, half8v* hi, half8v* lo) {
 #pragma unroll
     for (int t = 0; t < 8; t += 2) {
         const float2v p = {v[t], v[t + 1]};
         const half2v h = __builtin_convertvector(p, half2v);
-        const float2v r = {v[t] - (float)h[0], v[t + 1] - (float)h[1]};
+        const float2v r = {__builtin_fmaf(v[t], one, -(float)h[0]), __builtin_fmaf(v[t + 1], one, -(float)h[1])};
         const half2v l = __builtin_convertvector(r, half2v);
         (*hi)[t] = h[0];
         (*hi)[t + 1] = h[1];
@@ -427,7 +485,7 @@ __device__ __forceinline__ void f16_step(const float (&x2v)[8], const float (&ra
         for (int t = 0; t < 8; t++) {
             rv[t] = raw[g][t] * scale[g];
         }
-        split_f16x8(rv, &bhi[g], &blo[g]);
+        split_f16x8(rv, kc.one, &bhi[g], &blo[g]);
     }
 
 #pragma unroll
@@ -436,7 +494,7 @@ __device__ __forceinline__ void f16_step(const float (&x2v)[8], const float (&ra
 #pragma unroll
         for (int t = 0; t < 8; t += 2) {
             half2v h, l;
-            kernel_pair_f16<KT>(x1v[r], x2v[t], x2v[t + 1], kc, &h, &l);
+            kernel_pair_f16<KT>(x1v[r], x2v[t], x2v[t + 1], kc, kc.one, &h, &l);
             ahi[t] = h[0];
             ahi[t + 1] = h[1];
             alo[t] = l[0];
@@ -454,22 +512,13 @@ __device__ __forceinline__ void f16_step(const float (&x2v)[8], const float (&ra
 // PF: request the next step's operands before evaluating the current one (costs 8 + 8 G
 // registers; used for G = 1 where they are available).
 template <int KT, int G, int R, bool PF>
-__global__ void __launch_bounds__(512) fwd_mfma_f16(const FwdArgs a) {
-    extern __shared__ float lds[];
-
+__device__ __forceinline__ void fwd_mfma_f16_body(const FwdArgs& a, float* lds, const WaveView& w,
+                                                  int row0) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int S = blockDim.x >> 6;
     const int li = lane & 15;
     const int kk = lane >> 4;
-
-    const long long item = xcd_item(blockIdx.x, a.items_per_xcd);
-    if (item >= a.total_items) {
-        return;
-    }
-    int chunk_in_block;
-    const WaveView w = wave_view(a, item, a.chunks_per_block, &chunk_in_block);
-    const int row0 = w.row_block * KM_BLOCK_SIZE + chunk_in_block * (16 * R);
     const int kbase = blockIdx.y * (16 * G);
 
     const KernelConsts kc = make_consts<KT>(w.params, a.params_s, false);
@@ -563,6 +612,262 @@ __global__ void __launch_bounds__(512) fwd_mfma_f16(const FwdArgs a) {
     }
 }
 
+template <int KT, int G, int R, bool PF>
+__global__ void __launch_bounds__(512) fwd_mfma_f16(const FwdArgs a) {
+    extern __shared__ float lds[];
+    KM_TL_BEGIN();
+    const ItemRef it = decode_item(a);
+    if (!it.valid) {
+        return;
+    }
+    int chunk_in_block;
+    if constexpr (R == 8) {
+        if (it.small) {
+            const WaveView w = wave_view(a, it.item, 1, &chunk_in_block);
+            fwd_mfma_f16_body<KT, G, 1, false>(a, lds, w, w.row_block * KM_BLOCK_SIZE + 16 * it.piece);
+            KM_TL_END();
+            return;
+        }
+    }
+    const WaveView w = wave_view(a, it.item, a.chunks_per_block, &chunk_in_block);
+    fwd_mfma_f16_body<KT, G, R, PF>(a, lds, w, w.row_block * KM_BLOCK_SIZE + chunk_in_block * (16 * R));
+    KM_TL_END();
+}
+
+// ---------------------------------------------------------------------------------------
+// Spectral kernel, phase-split form of the split-fp16 variant.
+//
+// With a reference point c per wavefront (its first row) and A_i = 2 pi f (x1_i - c),
+// B_j = 2 pi f (x2_j - c):
+//     cos(2 pi f (x1_i - x2_j)) = cos A_i cos B_j + sin A_i sin B_j
+//     out[i,:] = cos A_i * sum_j E_ij (cos B_j rhs[j,:]) + sin A_i * sum_j E_ij (sin B_j rhs[j,:])
+// with E_ij = exp(-d^2 / (2 l^2)) the Gaussian factor alone.  The cosine leaves the per-pair
+// work: a pair costs sub, mul, fma, exp2 and the hi/lo split (5 full-rate + 1 transcendental
+// instructions instead of 7 + 2), in exchange for twice the fp16 MFMAs, which run beside the
+// VALU.  cos B_j / sin B_j are needed once per column: each chunk of 512 columns is tabulated
+// cooperatively by the wavefront (8 columns per lane) into LDS together with x2, and the
+// steps read their 8 columns back as broadcast vector reads.  Phases are formed as
+// fract(f * delta) with the rounding error of the product added back (one fma), so they are
+// accurate to ~1e-7 revolutions for any window width.
+// ---------------------------------------------------------------------------------------
+#define KM_PHASE_CHUNK 512
+
+__device__ __forceinline__ float phase_rev(float f, float delta) {
+    const float p = f * delta;
+    const float err = __builtin_fmaf(f, delta, -p);  // exact rounding error of the product
+    return __builtin_amdgcn_fractf(p) + err;
+}
+
+template <int G>
+__device__ __forceinline__ void rhs_load(const FwdArgs& a, const WaveView& w, int c0, int col_end,
+                                         int kk, const unsigned (&rhs_lane)[G], float (&raw)[G][8]) {
+    if (c0 + 32 <= col_end) {
+        const float* ru = w.rhs + (long long)c0 * a.rhs_s0;
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                raw[g][t] = (ru + t * a.rhs_s0)[rhs_lane[g]];
+            }
+        }
+    } else {
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+            const int col = c0 + 8 * kk + t;
+            const int colc = min(col, col_end - 1);
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                const float v = w.rhs[(long long)colc * a.rhs_s0 + (rhs_lane[g] - (unsigned)(8 * kk * a.rhs_s0))];
+                raw[g][t] = col < col_end ? v : 0.0f;
+            }
+        }
+    }
+}
+
+template <int G, int R, bool PF>
+__device__ __forceinline__ void fwd_spectral_f16_body(const FwdArgs& a, float* lds, const WaveView& w,
+                                                      int row0) {
+    constexpr int KT = KM_KERNEL_SPECTRAL;
+    constexpr int GE = 2 * G;  // accumulator groups: [cos part of g = 0..G) , sin part of g = 0..G)]
+    constexpr int CH = KM_PHASE_CHUNK;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int S = blockDim.x >> 6;
+    const int li = lane & 15;
+    const int kk = lane >> 4;
+    const int kbase = blockIdx.y * (16 * G);
+
+    const KernelConsts kc = make_consts<KT>(w.params, a.params_s, false);
+    const float sigma = w.params[KernelTraits<KT>::SIGMA * a.params_s];
+    const float c_ref = w.x1[(long long)min(row0, a.m - 1) * a.x1_s];
+
+    int col_begin = w.range_start;
+    int col_end = w.range_end;
+    if (S > 1) {
+        const int width = max(w.range_end - w.range_start, 0);
+        const int per_wave = ((width + S - 1) / S + 31) & ~31;
+        col_begin = w.range_start + wave * per_wave;
+        col_end = min(w.range_end, col_begin + per_wave);
+    }
+
+    float x1v[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int row = min(row0 + 16 * r + li, a.m - 1);
+        x1v[r] = w.x1[(long long)row * a.x1_s];
+    }
+
+    bool colmask[GE];
+    unsigned rhs_lane[G];
+    int shift[GE];
+    float scale[GE];
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        const int c = kbase + 16 * g + li;
+        rhs_lane[g] = (unsigned)(8 * kk * a.rhs_s0 + min(c, a.k - 1) * a.rhs_s1);
+#pragma unroll
+        for (int part = 0; part < 2; part++) {
+            colmask[part * G + g] = c < a.k;
+            shift[part * G + g] = 100;
+            scale[part * G + g] = c < a.k ? __builtin_ldexpf(1.0f, 100) : 0.0f;
+        }
+    }
+
+    float4v acc[R][GE];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+#pragma unroll
+        for (int g = 0; g < GE; g++) {
+            acc[r][g] = (float4v){0.0f, 0.0f, 0.0f, 0.0f};
+        }
+    }
+
+    // Per-wavefront table of the current chunk: x2, cos B, sin B.
+    float* tab_x2 = lds + (size_t)wave * (3 * CH);
+    float* tab_cos = tab_x2 + CH;
+    float* tab_sin = tab_cos + CH;
+    float* reduce_buffer = lds + (size_t)S * (3 * CH);
+
+    for (int chunk0 = col_begin; chunk0 < col_end; chunk0 += CH) {
+        const int chunk_end = min(chunk0 + CH, col_end);
+        const int padded = (chunk_end - chunk0 + 31) & ~31;
+        for (int q = lane; q < padded; q += 64) {
+            const int col = min(chunk0 + q, chunk_end - 1);
+            const float xv = w.x2[(long long)col * a.x2_s];
+            const float th = phase_rev(kc.f, xv - c_ref);
+            tab_x2[q] = xv;
+            tab_cos[q] = __builtin_amdgcn_cosf(th);
+            tab_sin[q] = __builtin_amdgcn_sinf(th);
+        }
+        // The table is written and read by this wavefront only.
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+        float raw[G][8];
+        rhs_load<G>(a, w, chunk0, chunk_end, kk, rhs_lane, raw);
+        for (int c0 = chunk0; c0 < chunk_end; c0 += 32) {
+            const bool more = c0 + 32 < chunk_end;
+            float rawn[G][8];
+            if (PF && more) {
+                rhs_load<G>(a, w, c0 + 32, chunk_end, kk, rhs_lane, rawn);
+            }
+            const int off = c0 - chunk0 + 8 * kk;
+            float x2v[8], cb[8], sb[8];
+#pragma unroll
+            for (int t = 0; t < 8; t += 4) {
+                const float4v vx = *(const float4v*)(tab_x2 + off + t);
+                const float4v vc = *(const float4v*)(tab_cos + off + t);
+                const float4v vs = *(const float4v*)(tab_sin + off + t);
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    x2v[t + u] = vx[u];
+                    cb[t + u] = vc[u];
+                    sb[t + u] = vs[u];
+                }
+            }
+            float braw[GE][8];
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+#pragma unroll
+                for (int t = 0; t < 8; t++) {
+                    braw[g][t] = raw[g][t] * cb[t];
+                    braw[G + g][t] = raw[g][t] * sb[t];
+                }
+            }
+            f16_step<KM_KERNEL_RBF, GE, R>(x2v, braw, x1v, kc, colmask, shift, scale, acc);
+            if (more) {
+                if (PF) {
+#pragma unroll
+                    for (int g = 0; g < G; g++) {
+#pragma unroll
+                        for (int t = 0; t < 8; t++) {
+                            raw[g][t] = rawn[g][t];
+                        }
+                    }
+                } else {
+                    rhs_load<G>(a, w, c0 + 32, chunk_end, kk, rhs_lane, raw);
+                }
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    }
+
+    // out = sigma * (cos A * P + sin A * Q) with the power-of-two scales undone; A for the rows
+    // this lane holds in the accumulator layout.
+    float4v res[R][G];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        float ca[4], sa[4];
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            const int row = min(row0 + 16 * r + 4 * kk + v, a.m - 1);
+            const float th = phase_rev(kc.f, w.x1[(long long)row * a.x1_s] - c_ref);
+            ca[v] = __builtin_amdgcn_cosf(th);
+            sa[v] = __builtin_amdgcn_sinf(th);
+        }
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            const float up = __builtin_ldexpf(sigma, -shift[g] - KM_F16_KSCALE_LOG2);
+            const float uq = __builtin_ldexpf(sigma, -shift[G + g] - KM_F16_KSCALE_LOG2);
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                res[r][g][v] = ca[v] * (acc[r][g][v] * up) + sa[v] * (acc[r][G + g][v] * uq);
+            }
+        }
+    }
+    float* __restrict__ out = a.out + w.b * (long long)a.m * a.k;
+    if (S == 1) {
+        store_direct<G, R>(res, lane, out, row0, kbase, a.m, a.k);
+    } else {
+        reduce_and_store<G, R>(res, reduce_buffer, S, wave, lane, out, row0, kbase, a.m, a.k);
+    }
+}
+
+template <int G, int R, bool PF>
+__global__ void __launch_bounds__(512) fwd_spectral_f16(const FwdArgs a) {
+    extern __shared__ float lds[];
+    KM_TL_BEGIN();
+    const ItemRef it = decode_item(a);
+    if (!it.valid) {
+        return;
+    }
+    int chunk_in_block;
+    if constexpr (R == 8) {
+        if (it.small) {
+            const WaveView w = wave_view(a, it.item, 1, &chunk_in_block);
+            fwd_spectral_f16_body<G, 1, false>(a, lds, w, w.row_block * KM_BLOCK_SIZE + 16 * it.piece);
+            KM_TL_END();
+            return;
+        }
+    }
+    const WaveView w = wave_view(a, it.item, a.chunks_per_block, &chunk_in_block);
+    fwd_spectral_f16_body<G, R, PF>(a, lds, w, w.row_block * KM_BLOCK_SIZE + chunk_in_block * (16 * R));
+    KM_TL_END();
+}
+
 // ---------------------------------------------------------------------------------------
 // VALU variant: one workgroup of two wavefronts per 128-row block, one row per lane,
 // KC rhs columns per pass.  x2[j] and rhs[j][0..KC) are the same for every lane, so they
@@ -630,7 +935,16 @@ template <int KT, int G, int R>
 static hipError_t launch_mfma(const FwdArgs& a, int variant, int S, unsigned gx, unsigned gy,
                               hipStream_t stream) {
     const size_t lds = S > 1 ? (size_t)S * R * G * 4 * 64 * sizeof(float) : 0;
-    if (variant == KM_VARIANT_MFMA_F16) {
+    if (variant == KM_VARIANT_MFMA_F16 && KT == KM_KERNEL_SPECTRAL) {
+        // Instantiated only for the shapes the launch table can pick (register budget).
+        if constexpr (G * R <= 8) {
+            const size_t table = (size_t)S * 3 * KM_PHASE_CHUNK * sizeof(float);
+            hipLaunchKernelGGL((fwd_spectral_f16<G, R, false>), dim3(gx, gy, 1),
+                               dim3(64 * S, 1, 1), table + lds, stream, a);
+        } else {
+            return hipErrorInvalidConfiguration;
+        }
+    } else if (variant == KM_VARIANT_MFMA_F16 || variant == KM_VARIANT_MFMA_F16_DIRECT) {
         hipLaunchKernelGGL((fwd_mfma_f16<KT, G, R, G == 1>), dim3(gx, gy, 1), dim3(64 * S, 1, 1), lds, stream, a);
     } else {
         hipLaunchKernelGGL((fwd_mfma_f32<KT, G, R>), dim3(gx, gy, 1), dim3(64 * S, 1, 1), lds, stream, a);
@@ -707,8 +1021,17 @@ hipError_t launch_matmul(const MatmulProblem& p, const MatmulPlan& plan, hipStre
         a.total_items = row_blocks * a.chunks_per_block * p.num_batches;
     }
     a.items_per_xcd = (a.total_items + KM_NUM_XCD - 1) / KM_NUM_XCD;
-    const unsigned grid_x = (unsigned)(a.items_per_xcd * KM_NUM_XCD);
+    a.tail_items = 0;
+    unsigned grid_x = (unsigned)(a.items_per_xcd * KM_NUM_XCD);
     const unsigned grid_y = (unsigned)((p.k + plan.k_chunk - 1) / plan.k_chunk);
+    // Tail balancing (split-fp16 kernels, one wavefront per 128-row block): whatever does not
+    // fill all 128 SIMDs of an XCD evenly is cut into 16-row pieces and dispatched last.
+    const bool f16 = plan.variant == KM_VARIANT_MFMA_F16 || plan.variant == KM_VARIANT_MFMA_F16_DIRECT;
+    if (f16 && plan.row_groups == 8 && plan.col_splits == 1 && plan.tail_balance &&
+        a.items_per_xcd >= 2 * 128) {
+        a.tail_items = (int)(a.items_per_xcd % 128);
+        grid_x = (unsigned)((a.items_per_xcd - a.tail_items + 8LL * a.tail_items) * KM_NUM_XCD);
+    }
 
     if (plan.variant == KM_VARIANT_VALU) {
         switch (p.kernel_type) {

@@ -48,7 +48,8 @@ def test_matmul(example_data, col_blocks):
 
 
 @pytest.mark.parametrize("variant,rows", [("valu", None), ("mfma_f32", 16), ("mfma_f32", 32), ("mfma_f32", 64), ("mfma_f32", 128),
-                                          ("mfma_f16", 16), ("mfma_f16", 32), ("mfma_f16", 64), ("mfma_f16", 128)])
+                                          ("mfma_f16", 16), ("mfma_f16", 32), ("mfma_f16", 64), ("mfma_f16", 128),
+                                          ("mfma_f16_direct", 32), ("mfma_f16_direct", 128)])
 def test_matmul_variants(example_data, variant, rows):
     d = example_data
     args = (d.x1, d.x2, d.rhs, d.params, d.start, d.end)
