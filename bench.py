@@ -83,6 +83,7 @@ def main() -> int:
     ap.add_argument("--rows-per-wave", type=int, default=0)
     ap.add_argument("--col-splits", type=int, default=0)
     ap.add_argument("--batch", type=int, default=None, help="override the number of batch items")
+    ap.add_argument("--no-tail-balance", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB elementwise add-scalar (a copy-like kernel of known traffic "
@@ -137,6 +138,8 @@ def main() -> int:
         defines["MATMUL_ROWS_PER_WAVE"] = args.rows_per_wave
     if args.col_splits:
         defines["MATMUL_COL_BLOCKS"] = args.col_splits
+    if args.no_tail_balance:
+        defines["MATMUL_TAIL_BALANCE"] = 0
     op = load_native("matmul", defines)
     if is_grad:
         from kernel_matmul_amd.configurations import BilinearDerivativeConfiguration

@@ -46,6 +46,14 @@ __device__ unsigned long long* g_timeline;
 #define KM_TL_END()
 #endif
 
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ half8v join_half2x4(const half2v (&p)[4]) {
+    const half4v a = __builtin_shufflevector(p[0], p[1], 0, 1, 2, 3);
+    const half4v b = __builtin_shufflevector(p[2], p[3], 0, 1, 2, 3);
+    return __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
 struct FwdArgs {
     BatchShape batch;
     long long num_batches;
@@ -363,7 +371,7 @@ template <int KT>
 __device__ __forceinline__ void kernel_pair_f16(float x1, float x2a, float x2b, const KernelConsts& c,
                                                 float one, half2v* hi, half2v* lo) {
     // Two neighbouring columns at once so that the conversions pack.
-    float2v kv, res;
+    float2v kv;
     float ea[2], ca[2];
     const float x2s[2] = {x2a, x2b};
 #pragma unroll
@@ -386,29 +394,29 @@ __device__ __forceinline__ void kernel_pair_f16(float x1, float x2a, float x2b, 
         kv[t] = KT == KM_KERNEL_SPECTRAL ? ea[t] * ca[t] : ea[t];
     }
     const half2v h = __builtin_convertvector(kv, half2v);
+    half2v l;
 #pragma unroll
     for (int t = 0; t < 2; t++) {
-        // Residual of the exact product where there is one (contracts to one fused op).
-        // Written as fma so that it maps to one v_fma_mix_f32 (fp16 operand read directly);
-        // `one` is a run-time 1.0 the compiler cannot fold away.
-        res[t] = __builtin_fmaf(ea[t], KT == KM_KERNEL_SPECTRAL ? ca[t] : one, -(float)h[t]);
+        // Residual of the exact product where there is one, computed and rounded to fp16 by
+        // one v_fma_mixlo/hi_f16 (the fp16 operand is read directly).  `one` is a run-time
+        // 1.0 that keeps the expression an fma.
+        l[t] = (_Float16)__builtin_fmaf(ea[t], KT == KM_KERNEL_SPECTRAL ? ca[t] : one, -(float)h[t]);
     }
     *hi = h;
-    *lo = __builtin_convertvector(res, half2v);
+    *lo = l;
 }
 
 __device__ __forceinline__ void split_f16x8(const float (&v)[8], float one, half8v* hi, half8v* lo) {
+    half2v h2[4], l2[4];
 #pragma unroll
-    for (int t = 0; t < 8; t += 2) {
-        const float2v p = {v[t], v[t + 1]};
-        const half2v h = __builtin_convertvector(p, half2v);
-        const float2v r = {__builtin_fmaf(v[t], one, -(float)h[0]), __builtin_fmaf(v[t + 1], one, -(float)h[1])};
-        const half2v l = __builtin_convertvector(r, half2v);
-        (*hi)[t] = h[0];
-        (*hi)[t + 1] = h[1];
-        (*lo)[t] = l[0];
-        (*lo)[t + 1] = l[1];
+    for (int t = 0; t < 4; t++) {
+        const float2v p = {v[2 * t], v[2 * t + 1]};
+        h2[t] = __builtin_convertvector(p, half2v);
+        l2[t][0] = (_Float16)__builtin_fmaf(v[2 * t], one, -(float)h2[t][0]);
+        l2[t][1] = (_Float16)__builtin_fmaf(v[2 * t + 1], one, -(float)h2[t][1]);
     }
+    *hi = join_half2x4(h2);
+    *lo = join_half2x4(l2);
 }
 
 // Operands of one step of 32 columns for this lane: x2 and rhs at columns c0 + 8 kk + t.
@@ -490,16 +498,13 @@ __device__ __forceinline__ void f16_step(const float (&x2v)[8], const float (&ra
 
 #pragma unroll
     for (int r = 0; r < R; r++) {
-        half8v ahi, alo;
+        half2v h2[4], l2[4];
 #pragma unroll
-        for (int t = 0; t < 8; t += 2) {
-            half2v h, l;
-            kernel_pair_f16<KT>(x1v[r], x2v[t], x2v[t + 1], kc, kc.one, &h, &l);
-            ahi[t] = h[0];
-            ahi[t + 1] = h[1];
-            alo[t] = l[0];
-            alo[t + 1] = l[1];
+        for (int t = 0; t < 4; t++) {
+            kernel_pair_f16<KT>(x1v[r], x2v[2 * t], x2v[2 * t + 1], kc, kc.one, &h2[t], &l2[t]);
         }
+        const half8v ahi = join_half2x4(h2);
+        const half8v alo = join_half2x4(l2);
 #pragma unroll
         for (int g = 0; g < G; g++) {
             acc[r][g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahi, bhi[g], acc[r][g], 0, 0, 0);
@@ -937,7 +942,7 @@ static hipError_t launch_mfma(const FwdArgs& a, int variant, int S, unsigned gx,
     const size_t lds = S > 1 ? (size_t)S * R * G * 4 * 64 * sizeof(float) : 0;
     if (variant == KM_VARIANT_MFMA_F16 && KT == KM_KERNEL_SPECTRAL) {
         // Instantiated only for the shapes the launch table can pick (register budget).
-        if constexpr (G * R <= 8) {
+        if constexpr (G == 1) {
             const size_t table = (size_t)S * 3 * KM_PHASE_CHUNK * sizeof(float);
             hipLaunchKernelGGL((fwd_spectral_f16<G, R, false>), dim3(gx, gy, 1),
                                dim3(64 * S, 1, 1), table + lds, stream, a);
