@@ -106,7 +106,8 @@ class NativeModule:
             options.col_splits = max(s for s in (1, 2, 4, 8) if s <= col_blocks)
         variant = self.defines.get("MATMUL_VARIANT")
         if variant is not None:
-            options.variant = {"auto": 0, "valu": 1, "mfma": 2, "mfma_f32": 2, "mfma_f16": 3, "mfma_f16_direct": 4}[variant]
+            options.variant = {"auto": 0, "valu": 1, "mfma": 2, "mfma_f32": 2, "mfma_f16": 3, "mfma_f16_direct": 4,
+                               "block": 5}[variant]
         if self.defines.get("MATMUL_TAIL_BALANCE") == 0:
             options.reserved = 1
         rows = self.defines.get("MATMUL_ROWS_PER_WAVE")

@@ -83,12 +83,26 @@ static const long long TARGET_WAVES = 4096;
 
 static int make_plan(const MatmulProblem& p, const km_launch_options* opt, MatmulPlan* plan) {
     int variant = opt ? opt->variant : KM_VARIANT_AUTO;
+    plan->phase_split = 0;
     if (variant == KM_VARIANT_AUTO) {
         variant = KM_VARIANT_MFMA_F16;
     }
     if (variant != KM_VARIANT_VALU && variant != KM_VARIANT_MFMA_F32 && variant != KM_VARIANT_MFMA_F16 &&
-        variant != KM_VARIANT_MFMA_F16_DIRECT) {
+        variant != KM_VARIANT_MFMA_F16_DIRECT && variant != KM_VARIANT_BLOCK) {
         return fail(KM_ERR_INVALID_ARGUMENT, "km_matmul: unknown variant %d", variant);
+    }
+    if (variant == KM_VARIANT_BLOCK) {
+        if (opt && (opt->rows_per_wave != 0 || opt->col_splits > 1)) {
+            return fail(KM_ERR_INVALID_ARGUMENT,
+                        "km_matmul: the workgroup-shared variant has a fixed decomposition");
+        }
+        plan->variant = variant;
+        plan->k_chunk = p.k <= 16 ? 16 : 32;
+        plan->row_groups = 8;
+        plan->col_splits = 1;
+        plan->tail_balance = !(opt && opt->reserved == 1);
+        plan->phase_split = p.kernel_type == KM_KERNEL_SPECTRAL && p.k <= 16;
+        return KM_OK;
     }
     plan->variant = variant;
     if (variant == KM_VARIANT_VALU) {

@@ -12,7 +12,8 @@ enum {
     KM_VARIANT_VALU = 1,
     KM_VARIANT_MFMA_F32 = 2,
     KM_VARIANT_MFMA_F16 = 3,         // split-fp16 MFMA; spectral kernels in phase-split form
-    KM_VARIANT_MFMA_F16_DIRECT = 4   // split-fp16 MFMA with the cosine evaluated per pair
+    KM_VARIANT_MFMA_F16_DIRECT = 4,  // split-fp16 MFMA with the cosine evaluated per pair
+    KM_VARIANT_BLOCK = 5             // split-fp16 MFMA, rhs operand prepared once per workgroup of 4 row blocks
 };
 
 struct MatmulProblem {
@@ -43,9 +44,11 @@ struct MatmulPlan {
     int row_groups;  // MFMA: groups of 16 rows per wavefront (1, 2, 4, 8)
     int col_splits;  // MFMA: wavefronts per workgroup sharing one column range (1, 2, 4, 8)
     int tail_balance;  // split-fp16 kernels: cut the uneven remainder into 16-row pieces
+    int phase_split;   // KM_VARIANT_BLOCK: spectral kernel in phase-split form
 };
 
 hipError_t launch_matmul(const MatmulProblem& p, const MatmulPlan& plan, hipStream_t stream);
+hipError_t launch_matmul_block(const MatmulProblem& p, const MatmulPlan& plan, hipStream_t stream);
 
 struct ParamGradProblem {
     int kernel_type;

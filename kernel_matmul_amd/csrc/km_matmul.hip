@@ -18,13 +18,11 @@
 // range.
 #include "km_batch.h"
 #include "km_common.h"
+#include "km_fwd.h"
 #include "km_launch.h"
 
 namespace km {
 
-typedef _Float16 half8v __attribute__((ext_vector_type(8)));
-typedef _Float16 half2v __attribute__((ext_vector_type(2)));
-typedef float float2v __attribute__((ext_vector_type(2)));
 
 #ifdef KM_TIMELINE
 // Development aid (never defined in the library build): per-wavefront placement and
@@ -46,32 +44,7 @@ __device__ unsigned long long* g_timeline;
 #define KM_TL_END()
 #endif
 
-typedef _Float16 half4v __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ half8v join_half2x4(const half2v (&p)[4]) {
-    const half4v a = __builtin_shufflevector(p[0], p[1], 0, 1, 2, 3);
-    const half4v b = __builtin_shufflevector(p[2], p[3], 0, 1, 2, 3);
-    return __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
-}
-
-struct FwdArgs {
-    BatchShape batch;
-    long long num_batches;
-    long long total_items;   // row chunks * batches
-    long long items_per_xcd;
-    int m, n, k;
-    int chunks_per_block;    // 128 / rows per workgroup
-    int tail_items;          // per XCD: row-block items at the end that are split 8 ways by rows
-    const float* x1;
-    const float* x2;
-    const float* rhs;
-    const float* params;
-    const int* start;
-    const int* end;
-    float* out;
-    BatchStrides x1_bs, x2_bs, rhs_bs, params_bs, start_bs, end_bs;
-    long long x1_s, x2_s, rhs_s0, rhs_s1, params_s, start_s, end_s;
-};
 
 // Per-wavefront view of the problem, shared by the three kernels.
 struct WaveView {
@@ -365,7 +338,6 @@ __global__ void __launch_bounds__(512) fwd_mfma_f32(const FwdArgs a) {
 //     accumulators are multiplied by the (exact) ratio, so no pass over rhs is needed.
 // Both scales and sigma are undone on the accumulators before they leave the wavefront.
 // ---------------------------------------------------------------------------------------
-#define KM_F16_KSCALE_LOG2 14
 
 template <int KT>
 __device__ __forceinline__ void kernel_pair_f16(float x1, float x2a, float x2b, const KernelConsts& c,
@@ -651,17 +623,12 @@ __global__ void __launch_bounds__(512) fwd_mfma_f16(const FwdArgs a) {
 // instructions instead of 7 + 2), in exchange for twice the fp16 MFMAs, which run beside the
 // VALU.  cos B_j / sin B_j are needed once per column: each chunk of 512 columns is tabulated
 // cooperatively by the wavefront (8 columns per lane) into LDS together with x2, and the
-// steps read their 8 columns back as broadcast vector reads.  Phases are formed as
-// fract(f * delta) with the rounding error of the product added back (one fma), so they are
-// accurate to ~1e-7 revolutions for any window width.
+// steps read their 8 columns back as broadcast vector reads.  Phases are formed in double
+// precision (once per row / column), so they are accurate to 3e-8 revolutions for any window
+// width.
 // ---------------------------------------------------------------------------------------
 #define KM_PHASE_CHUNK 512
 
-__device__ __forceinline__ float phase_rev(float f, float delta) {
-    const float p = f * delta;
-    const float err = __builtin_fmaf(f, delta, -p);  // exact rounding error of the product
-    return __builtin_amdgcn_fractf(p) + err;
-}
 
 template <int G>
 __device__ __forceinline__ void rhs_load(const FwdArgs& a, const WaveView& w, int c0, int col_end,
@@ -760,7 +727,7 @@ __device__ __forceinline__ void fwd_spectral_f16_body(const FwdArgs& a, float* l
         for (int q = lane; q < padded; q += 64) {
             const int col = min(chunk0 + q, chunk_end - 1);
             const float xv = w.x2[(long long)col * a.x2_s];
-            const float th = phase_rev(kc.f, xv - c_ref);
+            const float th = phase_rev(kc.f, xv, c_ref);
             tab_x2[q] = xv;
             tab_cos[q] = __builtin_amdgcn_cosf(th);
             tab_sin[q] = __builtin_amdgcn_sinf(th);
@@ -829,7 +796,7 @@ __device__ __forceinline__ void fwd_spectral_f16_body(const FwdArgs& a, float* l
 #pragma unroll
         for (int v = 0; v < 4; v++) {
             const int row = min(row0 + 16 * r + 4 * kk + v, a.m - 1);
-            const float th = phase_rev(kc.f, w.x1[(long long)row * a.x1_s] - c_ref);
+            const float th = phase_rev(kc.f, w.x1[(long long)row * a.x1_s], c_ref);
             ca[v] = __builtin_amdgcn_cosf(th);
             sa[v] = __builtin_amdgcn_sinf(th);
         }
@@ -991,8 +958,8 @@ static hipError_t launch_valu(const FwdArgs& a, int KC, unsigned gx, unsigned gy
     return hipGetLastError();
 }
 
-hipError_t launch_matmul(const MatmulProblem& p, const MatmulPlan& plan, hipStream_t stream) {
-    FwdArgs a;
+void fill_fwd_args(const MatmulProblem& p, FwdArgs* args) {
+    FwdArgs& a = *args;
     const int r = p.batch_rank;
     const int64_t* const strides[6] = {p.x1_strides, p.x2_strides, p.rhs_strides,
                                        p.params_strides, p.start_strides, p.end_strides};
@@ -1016,6 +983,18 @@ hipError_t launch_matmul(const MatmulProblem& p, const MatmulPlan& plan, hipStre
     a.params_s = p.params_strides[r];
     a.start_s = p.start_strides[r];
     a.end_s = p.end_strides[r];
+    a.total_items = 0;
+    a.items_per_xcd = 0;
+    a.chunks_per_block = 1;
+    a.tail_items = 0;
+}
+
+hipError_t launch_matmul(const MatmulProblem& p, const MatmulPlan& plan, hipStream_t stream) {
+    if (plan.variant == KM_VARIANT_BLOCK) {
+        return launch_matmul_block(p, plan, stream);
+    }
+    FwdArgs a;
+    fill_fwd_args(p, &a);
 
     const long long row_blocks = (p.m + KM_BLOCK_SIZE - 1) / KM_BLOCK_SIZE;
     if (plan.variant == KM_VARIANT_VALU) {

@@ -67,10 +67,11 @@ def _matmul(kernel, a, rhs=None, variant=None):
     return load_native("matmul", defines).call(*op_args)
 
 
-@pytest.mark.parametrize("name", ["c2", "c3_rbf", "headline", "c5"])
-def test_forward_sampled_blocks_against_oracle(name):
+@pytest.mark.parametrize("name,variant", [("c2", None), ("c3_rbf", None), ("headline", None), ("c5", None),
+                                          ("c3_rbf", "block"), ("headline", "block"), ("c5", "block")])
+def test_forward_sampled_blocks_against_oracle(name, variant):
     kernel, n, batch, k, a, h = _build(name)
-    out = _matmul(kernel, a)
+    out = _matmul(kernel, a, variant=variant)
     assert out.shape == (batch, n, k)
     blocks = np.unique(np.concatenate([[0, 1, len(h["start"]) - 1],
                                        np.random.default_rng(1).integers(0, len(h["start"]), 5)]))

@@ -49,7 +49,7 @@ def test_matmul(example_data, col_blocks):
 
 @pytest.mark.parametrize("variant,rows", [("valu", None), ("mfma_f32", 16), ("mfma_f32", 32), ("mfma_f32", 64), ("mfma_f32", 128),
                                           ("mfma_f16", 16), ("mfma_f16", 32), ("mfma_f16", 64), ("mfma_f16", 128),
-                                          ("mfma_f16_direct", 32), ("mfma_f16_direct", 128)])
+                                          ("mfma_f16_direct", 32), ("mfma_f16_direct", 128), ("block", None)])
 def test_matmul_variants(example_data, variant, rows):
     d = example_data
     args = (d.x1, d.x2, d.rhs, d.params, d.start, d.end)
@@ -61,6 +61,52 @@ def test_matmul_variants(example_data, variant, rows):
     a = d.numpy()
     expected = oracle.matmul(d.kernel_type, a["x1"], a["x2"], a["rhs"], a["params"], a["start"], a["end"])
     assert_close(result, expected)
+
+
+@pytest.mark.parametrize("variant", ["auto", "block", "mfma_f16_direct", "mfma_f32"])
+def test_matmul_rhs_dynamic_range(example_data, variant):
+    """rhs whose magnitude spans 12 decades across columns and e^24 along the rows: the
+    half-precision contraction rescales its operands per column while it walks a row range, so
+    results must stay within the usual accumulation bound atol * |K| @ |rhs| everywhere.  The
+    half-precision variants represent K / sigma to an absolute 2^-39 (its low half underflows
+    below that), which adds the floor 2^-37 * sigma * sum |rhs| over the row's range; it only
+    shows when entries of K near zero meet rhs values many decades above the rest.  The
+    workgroup-shared variant scales rhs once for four row blocks, so its floor runs over the
+    union of their ranges."""
+    d = example_data
+    n, k = d.rhs.shape[-2], d.rhs.shape[-1]
+    col_scale = 10.0 ** torch.linspace(-6, 6, k, device=d.rhs.device)
+    if n % 2 == 0:
+        row_scale = torch.exp(torch.linspace(-12, 12, n, device=d.rhs.device))
+    else:  # odd sizes: magnitude falls along the rows, then jumps back up
+        row_scale = torch.exp(-torch.remainder(torch.linspace(0, 48, n, device=d.rhs.device), 24.0) + 12)
+    rhs = (d.rhs * col_scale * row_scale[:, None]).contiguous()
+    args = (d.x1, d.x2, rhs, d.params, d.start, d.end)
+    defines = MatmulSingleConfiguration(d.kernel_type).make_config(args)
+    defines["MATMUL_VARIANT"] = variant
+    result = load_native("matmul", defines).call(*args).detach().cpu().double().numpy()
+    a = d.numpy()
+    rhs64 = rhs.detach().cpu().double().numpy()
+    kd = oracle.dense(d.kernel_type, a["x1"], a["x2"], a["params"], a["start"], a["end"])
+    expected = kd @ rhs64
+    bound = np.abs(kd) @ np.abs(rhs64)
+    floor = 0.0
+    if variant != "mfma_f32":
+        start, end = a["start"].copy(), a["end"].copy()
+        if variant == "block":
+            for g0 in range(0, start.shape[-1], 4):
+                s_blk, e_blk = start[..., g0:g0 + 4], end[..., g0:g0 + 4]
+                empty = s_blk >= e_blk
+                lo = np.where(empty, np.iinfo(np.int32).max, s_blk).min(axis=-1, keepdims=True)
+                hi = np.where(empty, 0, e_blk).max(axis=-1, keepdims=True)
+                start[..., g0:g0 + 4], end[..., g0:g0 + 4] = np.minimum(lo, hi), hi
+        mask = oracle.range_mask(start, end, kd.shape[-2], kd.shape[-1])
+        sigma = np.abs(a["params"][..., -1, None, None])
+        floor = 2.0 ** -37 * sigma * (mask.astype(np.float64) @ np.abs(rhs64))
+    err = np.abs(result - expected)
+    assert np.all(np.isfinite(result))
+    tol = RTOL * np.abs(expected) + ATOL * bound + floor + 1e-30
+    assert np.all(err <= tol), float(np.max(err / tol))
 
 
 def _grad_tolerance(expected):
