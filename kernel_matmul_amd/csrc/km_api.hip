@@ -158,8 +158,8 @@ static int make_plan(const MatmulProblem& p, const km_launch_options* opt, Matmu
         }
     }
     // LDS per workgroup must stay within 64 KiB: the cross-wavefront reduction buffer takes
-    // S * R * G KiB and the phase-split kernel's tables 6 KiB per wavefront.
-    while (S > 1 && S * (R * G + (phase_split ? 6 : 0)) > 64) {
+    // S * R * G KiB and the phase-split kernel's tables 8.1 KiB per wavefront.
+    while (S > 1 && S * (R * G + (phase_split ? 9 : 0)) > 64) {
         S /= 2;
     }
     plan->row_groups = R;

@@ -45,13 +45,18 @@ void fill_fwd_args(const MatmulProblem& p, FwdArgs* args);
 // base-2 exponential) so that its hi and lo halves stay inside the fp16 exponent range.
 #define KM_F16_KSCALE_LOG2 14
 
-// Phase f * (x - c) in revolutions, reduced to [-0.5, 0.5].  It is needed once per row or column
-// (never per pair), so it is formed in double precision: neither the difference to the
-// reference point nor the product is rounded before the reduction, and the result carries
-// half an fp32 ulp of 0.5 (3e-8 revolutions) whatever the distance to c.
+// Phase f * (x - c) in revolutions, reduced to [-0.5, 0.5].  x - c is taken as an unevaluated
+// sum hi + lo (error-free transformation) and the product f * hi is never rounded on its own
+// (fused multiply-add), so the result carries about half an fp32 ulp of 0.5 (3e-8 revolutions) whatever the
+// distance to c — the accuracy of a double-precision evaluation at a third of its cost.
 __device__ __forceinline__ float phase_rev(float f, float x, float c) {
-    const double p = (double)f * ((double)x - (double)c);
-    return (float)(p - __builtin_rint(p));
+    const float hi = x - c;
+    const float bb = hi - x;
+    const float lo = (x - (hi - bb)) - (c + bb);
+    // f * hi - round(f * hi) in one fma (exact product, one rounding of a value within
+    // [-0.5, 0.5]), then the contribution of lo.
+    const float turns = __builtin_rintf(f * hi);
+    return __builtin_fmaf(f, lo, __builtin_fmaf(f, hi, -turns));
 }
 
 }  // namespace km

@@ -339,7 +339,9 @@ __global__ void __launch_bounds__(512) fwd_mfma_f32(const FwdArgs a) {
 // Both scales and sigma are undone on the accumulators before they leave the wavefront.
 // ---------------------------------------------------------------------------------------
 
-template <int KT>
+// FOLD: x1 holds x1 - r and x2a / x2b hold (x2 - r) * s for a common reference point r, so that
+// u = fma(x1, s, -x2) replaces subtract + multiply (used where both differences are exact).
+template <int KT, bool FOLD = false>
 __device__ __forceinline__ void kernel_pair_f16(float x1, float x2a, float x2b, const KernelConsts& c,
                                                 float one, half2v* hi, half2v* lo) {
     // Two neighbouring columns at once so that the conversions pack.
@@ -349,7 +351,7 @@ __device__ __forceinline__ void kernel_pair_f16(float x1, float x2a, float x2b, 
 #pragma unroll
     for (int t = 0; t < 2; t++) {
         const float d = x1 - x2s[t];
-        const float u = d * c.s;
+        const float u = FOLD ? __builtin_fmaf(x1, c.s, -x2s[t]) : d * c.s;
         const float arg = __builtin_fmaf(-u, u, (float)KM_F16_KSCALE_LOG2);
         if (KT == KM_KERNEL_RBF) {
             ea[t] = __builtin_amdgcn_exp2f(arg);
@@ -428,11 +430,11 @@ __device__ __forceinline__ void f16_load(const FwdArgs& a, const WaveView& w, in
 // One step of 32 columns: convert this lane's 8 rhs values per column group to hi/lo halves
 // (rescaling the accumulators first if a value would leave the fp16 range), then for every
 // row group evaluate 8 kernel entries, split them and issue the three MFMAs.
-template <int KT, int G, int R>
+template <int KT, int G, int R, bool FOLD = false>
 __device__ __forceinline__ void f16_step(const float (&x2v)[8], const float (&raw)[G][8],
                                          const float (&x1v)[R], const KernelConsts& kc,
                                          const bool (&colmask)[G], int (&shift)[G],
-                                         float (&scale)[G], float4v (&acc)[R][G]) {
+                                         float (&scale)[G], float4v (&acc)[R][G], float ref = 0.0f) {
     half8v bhi[G], blo[G];
 #pragma unroll
     for (int g = 0; g < G; g++) {
@@ -471,9 +473,10 @@ __device__ __forceinline__ void f16_step(const float (&x2v)[8], const float (&ra
 #pragma unroll
     for (int r = 0; r < R; r++) {
         half2v h2[4], l2[4];
+        const float x1 = FOLD ? x1v[r] - ref : x1v[r];  // FOLD: relative to the step's reference point
 #pragma unroll
         for (int t = 0; t < 4; t++) {
-            kernel_pair_f16<KT>(x1v[r], x2v[2 * t], x2v[2 * t + 1], kc, kc.one, &h2[t], &l2[t]);
+            kernel_pair_f16<KT, FOLD>(x1, x2v[2 * t], x2v[2 * t + 1], kc, kc.one, &h2[t], &l2[t]);
         }
         const half8v ahi = join_half2x4(h2);
         const half8v alo = join_half2x4(l2);
@@ -623,11 +626,12 @@ __global__ void __launch_bounds__(512) fwd_mfma_f16(const FwdArgs a) {
 // instructions instead of 7 + 2), in exchange for twice the fp16 MFMAs, which run beside the
 // VALU.  cos B_j / sin B_j are needed once per column: each chunk of 512 columns is tabulated
 // cooperatively by the wavefront (8 columns per lane) into LDS together with x2, and the
-// steps read their 8 columns back as broadcast vector reads.  Phases are formed in double
-// precision (once per row / column), so they are accurate to 3e-8 revolutions for any window
-// width.
+// steps read their 8 columns back as broadcast vector reads.  Phases are formed from an exact
+// two-term difference to the reference point (once per row / column), so they are accurate to
+// 3e-8 revolutions for any window width.
 // ---------------------------------------------------------------------------------------
 #define KM_PHASE_CHUNK 512
+#define KM_PHASE_TABLE_FLOATS (4 * KM_PHASE_CHUNK + KM_PHASE_CHUNK / 32) /* per wavefront */
 
 
 template <int G>
@@ -715,73 +719,131 @@ __device__ __forceinline__ void fwd_spectral_f16_body(const FwdArgs& a, float* l
         }
     }
 
-    // Per-wavefront table of the current chunk: x2, cos B, sin B.
-    float* tab_x2 = lds + (size_t)wave * (3 * CH);
+    // Per-wavefront table of the current chunk: x2, cos B, sin B, and for the folded form
+    // (x2 - r) * s with r the x2 value in the middle of each step of 32 columns.
+    float* tab_x2 = lds + (size_t)wave * KM_PHASE_TABLE_FLOATS;
     float* tab_cos = tab_x2 + CH;
     float* tab_sin = tab_cos + CH;
-    float* reduce_buffer = lds + (size_t)S * (3 * CH);
+    float* tab_xs = tab_sin + CH;
+    float* tab_ref = tab_xs + CH;
+    float* reduce_buffer = lds + (size_t)S * KM_PHASE_TABLE_FLOATS;
+
+    // Folded form u = fma(x1 - r, s, -[(x2 - r) s]): one instruction less per pair.  A chunk
+    // uses it only if it loses nothing: every x2 - r must be exact (error-free transformation),
+    // every x1 - r too (all coordinates involved are multiples of the ulp of the smallest
+    // magnitude, so a spread below that magnitude is sufficient), and |(x2 - r) s| <= 16 keeps
+    // the one rounding of the tabulated product below 1e-6.
+    float row_lo = __builtin_inff(), row_hi = -__builtin_inff();
+    bool row_nan = false;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        row_lo = fminf(row_lo, x1v[r]);
+        row_hi = fmaxf(row_hi, x1v[r]);
+        row_nan = row_nan || x1v[r] != x1v[r];
+    }
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        row_lo = fminf(row_lo, __shfl_xor(row_lo, off, 64));
+        row_hi = fmaxf(row_hi, __shfl_xor(row_hi, off, 64));
+    }
+    const bool rows_finite = !__any(row_nan);
+    row_lo = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, row_lo)));
+    row_hi = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, row_hi)));
 
     for (int chunk0 = col_begin; chunk0 < col_end; chunk0 += CH) {
         const int chunk_end = min(chunk0 + CH, col_end);
         const int padded = (chunk_end - chunk0 + 31) & ~31;
+        bool cols_ok = true;
+        float lo = row_lo, hi = row_hi;
+        // Strides are below 2^24 elements, so 32 x 32 -> 64 bit products are enough.
+        const float* x2c = w.x2 + (long long)chunk0 * a.x2_s;
+        const unsigned x2_stride = (unsigned)a.x2_s;
+        const int last = chunk_end - 1 - chunk0;
         for (int q = lane; q < padded; q += 64) {
-            const int col = min(chunk0 + q, chunk_end - 1);
-            const float xv = w.x2[(long long)col * a.x2_s];
+            const float xv = x2c[(unsigned long long)(unsigned)min(q, last) * x2_stride];
+            const float ref = x2c[(unsigned long long)(unsigned)min((q & ~31) + 16, last) * x2_stride];
+            const float xd = xv - ref;
+            const float bb = xd - xv;
+            const float err = (xv - (xd - bb)) - (ref + bb);  // exact rounding error of xd
+            const float xs = xd * kc.s;
             const float th = phase_rev(kc.f, xv, c_ref);
             tab_x2[q] = xv;
             tab_cos[q] = __builtin_amdgcn_cosf(th);
             tab_sin[q] = __builtin_amdgcn_sinf(th);
+            tab_xs[q] = xs;
+            if ((q & 31) == 0) {
+                tab_ref[q >> 5] = ref;
+            }
+            cols_ok = cols_ok && err == 0.0f && fabsf(xs) <= 16.0f;
+            lo = fminf(lo, ref);
+            hi = fmaxf(hi, ref);
         }
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            lo = fminf(lo, __shfl_xor(lo, off, 64));
+            hi = fmaxf(hi, __shfl_xor(hi, off, 64));
+        }
+        const bool rows_ok = rows_finite && (lo > 0.0f || hi < 0.0f) && (hi - lo) <= fminf(fabsf(lo), fabsf(hi));
+        const bool fold = __all(cols_ok) && rows_ok;
         // The table is written and read by this wavefront only.
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-        float raw[G][8];
-        rhs_load<G>(a, w, chunk0, chunk_end, kk, rhs_lane, raw);
-        for (int c0 = chunk0; c0 < chunk_end; c0 += 32) {
-            const bool more = c0 + 32 < chunk_end;
-            float rawn[G][8];
-            if (PF && more) {
-                rhs_load<G>(a, w, c0 + 32, chunk_end, kk, rhs_lane, rawn);
-            }
-            const int off = c0 - chunk0 + 8 * kk;
-            float x2v[8], cb[8], sb[8];
-#pragma unroll
-            for (int t = 0; t < 8; t += 4) {
-                const float4v vx = *(const float4v*)(tab_x2 + off + t);
-                const float4v vc = *(const float4v*)(tab_cos + off + t);
-                const float4v vs = *(const float4v*)(tab_sin + off + t);
-#pragma unroll
-                for (int u = 0; u < 4; u++) {
-                    x2v[t + u] = vx[u];
-                    cb[t + u] = vc[u];
-                    sb[t + u] = vs[u];
+        auto steps = [&](auto fold_c) {
+            constexpr bool FOLD = decltype(fold_c)::value;
+            float raw[G][8];
+            rhs_load<G>(a, w, chunk0, chunk_end, kk, rhs_lane, raw);
+            for (int c0 = chunk0; c0 < chunk_end; c0 += 32) {
+                const bool more = c0 + 32 < chunk_end;
+                float rawn[G][8];
+                if (PF && more) {
+                    rhs_load<G>(a, w, c0 + 32, chunk_end, kk, rhs_lane, rawn);
                 }
-            }
-            float braw[GE][8];
+                const int off = c0 - chunk0 + 8 * kk;
+                float x2v[8], cb[8], sb[8];
 #pragma unroll
-            for (int g = 0; g < G; g++) {
+                for (int t = 0; t < 8; t += 4) {
+                    const float4v vx = *(const float4v*)((FOLD ? tab_xs : tab_x2) + off + t);
+                    const float4v vc = *(const float4v*)(tab_cos + off + t);
+                    const float4v vs = *(const float4v*)(tab_sin + off + t);
 #pragma unroll
-                for (int t = 0; t < 8; t++) {
-                    braw[g][t] = raw[g][t] * cb[t];
-                    braw[G + g][t] = raw[g][t] * sb[t];
-                }
-            }
-            f16_step<KM_KERNEL_RBF, GE, R>(x2v, braw, x1v, kc, colmask, shift, scale, acc);
-            if (more) {
-                if (PF) {
-#pragma unroll
-                    for (int g = 0; g < G; g++) {
-#pragma unroll
-                        for (int t = 0; t < 8; t++) {
-                            raw[g][t] = rawn[g][t];
-                        }
+                    for (int u = 0; u < 4; u++) {
+                        x2v[t + u] = vx[u];
+                        cb[t + u] = vc[u];
+                        sb[t + u] = vs[u];
                     }
-                } else {
-                    rhs_load<G>(a, w, c0 + 32, chunk_end, kk, rhs_lane, raw);
+                }
+                const float ref = FOLD ? tab_ref[(c0 - chunk0) >> 5] : 0.0f;
+                float braw[GE][8];
+#pragma unroll
+                for (int g = 0; g < G; g++) {
+#pragma unroll
+                    for (int t = 0; t < 8; t++) {
+                        braw[g][t] = raw[g][t] * cb[t];
+                        braw[G + g][t] = raw[g][t] * sb[t];
+                    }
+                }
+                f16_step<KM_KERNEL_RBF, GE, R, FOLD>(x2v, braw, x1v, kc, colmask, shift, scale, acc, ref);
+                if (more) {
+                    if (PF) {
+#pragma unroll
+                        for (int g = 0; g < G; g++) {
+#pragma unroll
+                            for (int t = 0; t < 8; t++) {
+                                raw[g][t] = rawn[g][t];
+                            }
+                        }
+                    } else {
+                        rhs_load<G>(a, w, c0 + 32, chunk_end, kk, rhs_lane, raw);
+                    }
                 }
             }
+        };
+        if (fold) {
+            steps(std::integral_constant<bool, true>{});
+        } else {
+            steps(std::integral_constant<bool, false>{});
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -809,6 +871,9 @@ __device__ __forceinline__ void fwd_spectral_f16_body(const FwdArgs& a, float* l
                 res[r][g][v] = ca[v] * (acc[r][g][v] * up) + sa[v] * (acc[r][G + g][v] * uq);
             }
         }
+        // One row group at a time: keeps the double-precision phase arithmetic of several
+        // groups from being interleaved, which costs registers for nothing.
+        __builtin_amdgcn_sched_barrier(0);
     }
     float* __restrict__ out = a.out + w.b * (long long)a.m * a.k;
     if (S == 1) {
@@ -819,7 +884,7 @@ __device__ __forceinline__ void fwd_spectral_f16_body(const FwdArgs& a, float* l
 }
 
 template <int G, int R, bool PF>
-__global__ void __launch_bounds__(512) fwd_spectral_f16(const FwdArgs a) {
+__global__ void __launch_bounds__(512, 3) fwd_spectral_f16(const FwdArgs a) {
     extern __shared__ float lds[];
     KM_TL_BEGIN();
     const ItemRef it = decode_item(a);
@@ -910,7 +975,7 @@ static hipError_t launch_mfma(const FwdArgs& a, int variant, int S, unsigned gx,
     if (variant == KM_VARIANT_MFMA_F16 && KT == KM_KERNEL_SPECTRAL) {
         // Instantiated only for the shapes the launch table can pick (register budget).
         if constexpr (G == 1) {
-            const size_t table = (size_t)S * 3 * KM_PHASE_CHUNK * sizeof(float);
+            const size_t table = (size_t)S * KM_PHASE_TABLE_FLOATS * sizeof(float);
             hipLaunchKernelGGL((fwd_spectral_f16<G, R, false>), dim3(gx, gy, 1),
                                dim3(64 * S, 1, 1), table + lds, stream, a);
         } else {
