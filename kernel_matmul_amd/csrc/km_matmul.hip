@@ -851,16 +851,20 @@ __device__ __forceinline__ void fwd_spectral_f16_body(const FwdArgs& a, float* l
 
     // out = sigma * (cos A * P + sin A * Q) with the power-of-two scales undone; A for the rows
     // this lane holds in the accumulator layout.
+    // cos A / sin A are formed once per row by the lane that holds the row's coordinate
+    // (x1v: row 16 r + lane % 16) and fetched across lanes into the accumulator layout
+    // (rows 16 r + 4 (lane / 16) + v).
     float4v res[R][G];
 #pragma unroll
     for (int r = 0; r < R; r++) {
+        const float th = phase_rev(kc.f, x1v[r], c_ref);
+        const float ca_own = __builtin_amdgcn_cosf(th);
+        const float sa_own = __builtin_amdgcn_sinf(th);
         float ca[4], sa[4];
 #pragma unroll
         for (int v = 0; v < 4; v++) {
-            const int row = min(row0 + 16 * r + 4 * kk + v, a.m - 1);
-            const float th = phase_rev(kc.f, w.x1[(long long)row * a.x1_s], c_ref);
-            ca[v] = __builtin_amdgcn_cosf(th);
-            sa[v] = __builtin_amdgcn_sinf(th);
+            ca[v] = __shfl(ca_own, 4 * kk + v, 64);
+            sa[v] = __shfl(sa_own, 4 * kk + v, 64);
         }
 #pragma unroll
         for (int g = 0; g < G; g++) {

@@ -598,14 +598,18 @@ __global__ void __launch_bounds__(KM_BLK_THREADS, 3) fwd_block(const BlockArgs b
             continue;
         }
         const int row_base = (rb0 + r / 2) * KM_BLOCK_SIZE + 32 * wave + 16 * (r & 1) + 4 * kk;
+        // cos A / sin A: formed once per row by the lane that holds the row's coordinate
+        // (x1v: row 16 (r & 1) + lane % 16 of the 32), fetched across lanes into the accumulator
+        // layout (rows 4 (lane / 16) + v).
         float ca[4], sa[4];
         if (PHASE) {
+            const float th = phase_rev(kc.f, x1v[r], c_ref);
+            const float ca_own = __builtin_amdgcn_cosf(th);
+            const float sa_own = __builtin_amdgcn_sinf(th);
 #pragma unroll
             for (int v = 0; v < 4; v++) {
-                const int row = min(row_base + v, a.m - 1);
-                const float th = phase_rev(kc.f, x1[(long long)row * a.x1_s], c_ref);
-                ca[v] = __builtin_amdgcn_cosf(th);
-                sa[v] = __builtin_amdgcn_sinf(th);
+                ca[v] = __shfl(ca_own, 4 * kk + v, 64);
+                sa[v] = __shfl(sa_own, 4 * kk + v, 64);
             }
         }
 #pragma unroll
