@@ -74,12 +74,14 @@ static int check_common(const char* op, int kernel_type, int batch_rank, const i
     } while (0)
 
 // ---------------------------------------------------------------------------------------
-// gfx950 launch table for the forward operator.  256 CUs x 4 SIMDs: aim for at least four
-// wavefronts per SIMD.  Large problems run one wavefront per 128-row block (8 row groups,
+// gfx950 launch table for the forward operator.  256 CUs x 4 SIMDs: aim for at least one
+// wavefront per SIMD.  Large problems run one wavefront per 128-row block (8 row groups,
 // no cross-wavefront reduction); smaller ones first shrink the rows per wavefront, then
-// let several wavefronts share a row range.
+// let several wavefronts share a row range.  Fewer rows per wavefront repeat the rhs-operand
+// work and shared row ranges add a reduction, so neither goes further than filling the SIMDs
+// (measured: 1024 beats 2048 and 4096 from 157 to 3128 row-block items).
 // ---------------------------------------------------------------------------------------
-static const long long TARGET_WAVES = 4096;
+static const long long TARGET_WAVES = 1024;
 
 static int make_plan(const MatmulProblem& p, const km_launch_options* opt, MatmulPlan* plan) {
     int variant = opt ? opt->variant : KM_VARIANT_AUTO;
