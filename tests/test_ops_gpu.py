@@ -235,3 +235,54 @@ def test_index_bwd(example_data, shape):
             expected[b] += og[q] * grads[b + (slice(None), rows[q], cols[q])]
     err = np.abs(result.cpu().double().numpy() - expected)
     assert np.all(err <= _grad_tolerance(expected) + 1e-6), (result.cpu().numpy(), expected)
+
+
+# Coordinate regimes that decide between the folded evaluation u = fma(x1 - r, s, -(x2 - r) s)
+# and the plain (x1 - x2) s inside the split-fp16 kernels: the folded form is only taken where
+# both differences are exact in fp32, and either way results must meet the usual tolerance.
+COORDINATE_REGIMES = {
+    # name: (offset, extent, sorted)
+    "offset_1e5": (1.0e5, 150.0, True),      # coarse fp32 grid (ulp 2^-7): differences exact
+    "from_zero": (0.0, 150.0, True),         # first point exactly 0: spread > smallest magnitude
+    "negative": (-400.0, 150.0, True),       # all negative
+    "across_zero": (-75.0, 150.0, True),     # sign change inside the data
+    "tiny_offsets": (3.0, 1.0e-3, True),     # everything within one lengthscale
+    "unsorted_columns": (10.0, 20.0, False), # x2 in random order, full ranges
+}
+
+
+@pytest.mark.parametrize("variant", ["auto", "block"])
+@pytest.mark.parametrize("kernel_type", ["rbf", "spectral", "locally_periodic"])
+@pytest.mark.parametrize("regime", sorted(COORDINATE_REGIMES))
+def test_matmul_coordinate_regimes(regime, kernel_type, variant):
+    from kernel_matmul_amd.ranges import make_ranges
+    from tests.conftest import make_params
+
+    offset, extent, is_sorted = COORDINATE_REGIMES[regime]
+    g = torch.Generator().manual_seed(11)
+    m, k, batch = 1500, 16, (2,)
+    x = torch.rand(m, generator=g) * extent + offset
+    if is_sorted:
+        x = torch.sort(x)[0]
+        if regime == "from_zero":
+            x[0] = 0.0
+        x1 = x2 = x
+        start, end = make_ranges(2.5, x)
+    else:
+        x1 = torch.sort(x)[0]
+        x2 = x[torch.randperm(m, generator=g)]
+        rows = (m + 127) // 128
+        start = torch.zeros(rows, dtype=torch.int32)
+        end = torch.full((rows,), m, dtype=torch.int32)
+    rhs = torch.randn(m, k, generator=g)
+    rhs = rhs / torch.linalg.norm(rhs, dim=-2, keepdim=True)  # as the example data does
+    params = make_params(kernel_type, batch)
+    device = torch.device("cuda:0")
+    expand = lambda t: t.to(device).expand(*batch, *t.shape)
+    args = (expand(x1), expand(x2), expand(rhs), params.to(device), expand(start), expand(end))
+    defines = MatmulSingleConfiguration(kernel_type).make_config(args)
+    defines["MATMUL_VARIANT"] = variant
+    result = load_native("matmul", defines).call(*args)
+    f = lambda t: t.detach().cpu().numpy()
+    expected = oracle.matmul(kernel_type, *(f(t) for t in args))
+    assert_close(result, expected)
