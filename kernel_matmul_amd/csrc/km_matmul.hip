@@ -660,7 +660,7 @@ __device__ __forceinline__ void rhs_load(const FwdArgs& a, const WaveView& w, in
     }
 }
 
-template <int G, int R, bool PF>
+template <int G, int R>
 __device__ __forceinline__ void fwd_spectral_f16_body(const FwdArgs& a, float* lds, const WaveView& w,
                                                       int row0) {
     constexpr int KT = KM_KERNEL_SPECTRAL;
@@ -795,11 +795,6 @@ __device__ __forceinline__ void fwd_spectral_f16_body(const FwdArgs& a, float* l
             float raw[G][8];
             rhs_load<G>(a, w, chunk0, chunk_end, kk, rhs_lane, raw);
             for (int c0 = chunk0; c0 < chunk_end; c0 += 32) {
-                const bool more = c0 + 32 < chunk_end;
-                float rawn[G][8];
-                if (PF && more) {
-                    rhs_load<G>(a, w, c0 + 32, chunk_end, kk, rhs_lane, rawn);
-                }
                 const int off = c0 - chunk0 + 8 * kk;
                 float x2v[8], cb[8], sb[8];
 #pragma unroll
@@ -825,18 +820,8 @@ __device__ __forceinline__ void fwd_spectral_f16_body(const FwdArgs& a, float* l
                     }
                 }
                 f16_step<KM_KERNEL_RBF, GE, R, FOLD>(x2v, braw, x1v, kc, colmask, shift, scale, acc, ref);
-                if (more) {
-                    if (PF) {
-#pragma unroll
-                        for (int g = 0; g < G; g++) {
-#pragma unroll
-                            for (int t = 0; t < 8; t++) {
-                                raw[g][t] = rawn[g][t];
-                            }
-                        }
-                    } else {
-                        rhs_load<G>(a, w, c0 + 32, chunk_end, kk, rhs_lane, raw);
-                    }
+                if (c0 + 32 < chunk_end) {
+                    rhs_load<G>(a, w, c0 + 32, chunk_end, kk, rhs_lane, raw);
                 }
             }
         };
@@ -887,7 +872,7 @@ __device__ __forceinline__ void fwd_spectral_f16_body(const FwdArgs& a, float* l
     }
 }
 
-template <int G, int R, bool PF>
+template <int G, int R>
 __global__ void __launch_bounds__(512, 3) fwd_spectral_f16(const FwdArgs a) {
     extern __shared__ float lds[];
     KM_TL_BEGIN();
@@ -899,13 +884,13 @@ __global__ void __launch_bounds__(512, 3) fwd_spectral_f16(const FwdArgs a) {
     if constexpr (R == 8) {
         if (it.small) {
             const WaveView w = wave_view(a, it.item, 1, &chunk_in_block);
-            fwd_spectral_f16_body<G, 1, false>(a, lds, w, w.row_block * KM_BLOCK_SIZE + 16 * it.piece);
+            fwd_spectral_f16_body<G, 1>(a, lds, w, w.row_block * KM_BLOCK_SIZE + 16 * it.piece);
             KM_TL_END();
             return;
         }
     }
     const WaveView w = wave_view(a, it.item, a.chunks_per_block, &chunk_in_block);
-    fwd_spectral_f16_body<G, R, PF>(a, lds, w, w.row_block * KM_BLOCK_SIZE + chunk_in_block * (16 * R));
+    fwd_spectral_f16_body<G, R>(a, lds, w, w.row_block * KM_BLOCK_SIZE + chunk_in_block * (16 * R));
     KM_TL_END();
 }
 
@@ -980,13 +965,19 @@ static hipError_t launch_mfma(const FwdArgs& a, int variant, int S, unsigned gx,
         // Instantiated only for the shapes the launch table can pick (register budget).
         if constexpr (G == 1) {
             const size_t table = (size_t)S * KM_PHASE_TABLE_FLOATS * sizeof(float);
-            hipLaunchKernelGGL((fwd_spectral_f16<G, R, false>), dim3(gx, gy, 1),
+            hipLaunchKernelGGL((fwd_spectral_f16<G, R>), dim3(gx, gy, 1),
                                dim3(64 * S, 1, 1), table + lds, stream, a);
         } else {
             return hipErrorInvalidConfiguration;
         }
     } else if (variant == KM_VARIANT_MFMA_F16 || variant == KM_VARIANT_MFMA_F16_DIRECT) {
-        hipLaunchKernelGGL((fwd_mfma_f16<KT, G, R, G == 1>), dim3(gx, gy, 1), dim3(64 * S, 1, 1), lds, stream, a);
+        // Wide rhs tiles with many row groups exceed the register file; the launch table never
+        // picks them.
+        if constexpr (G * R <= 8) {
+            hipLaunchKernelGGL((fwd_mfma_f16<KT, G, R, G == 1>), dim3(gx, gy, 1), dim3(64 * S, 1, 1), lds, stream, a);
+        } else {
+            return hipErrorInvalidConfiguration;
+        }
     } else {
         hipLaunchKernelGGL((fwd_mfma_f32<KT, G, R>), dim3(gx, gy, 1), dim3(64 * S, 1, 1), lds, stream, a);
     }
