@@ -286,3 +286,69 @@ def test_matmul_coordinate_regimes(regime, kernel_type, variant):
     f = lambda t: t.detach().cpu().numpy()
     expected = oracle.matmul(kernel_type, *(f(t) for t in args))
     assert_close(result, expected)
+
+
+@pytest.mark.parametrize("variant", ["auto", "block", "mfma_f16_direct", "mfma_f32", "valu"])
+@pytest.mark.parametrize("kernel_type", ["rbf", "spectral"])
+def test_matmul_degenerate_ranges(kernel_type, variant):
+    """Row blocks with an empty range must produce exact zeros (the output is fully written),
+    ranges that reach past the last column are clipped (a symmetric pattern over fewer points
+    than one block reports end = block size > n, native/ranges/ranges.cpp:82-93), and single
+    rows / columns / rhs columns work."""
+    from tests.conftest import make_params
+
+    g = torch.Generator().manual_seed(5)
+    device = torch.device("cuda:0")
+    for m, n, k, start, end in [
+        (300, 300, 3, [0, 120, 290], [50, 120, 400]),   # partial, empty, clipped
+        (300, 300, 16, [10, 10, 10], [10, 10, 10]),     # all empty
+        (1, 1, 1, [0], [1]),
+        (129, 1, 2, [0, 0], [128, 1]),
+        (5, 700, 17, [3], [699]),
+    ]:
+        x1 = torch.sort(torch.rand(m, generator=g) * 10)[0]
+        x2 = torch.sort(torch.rand(n, generator=g) * 10)[0]
+        rhs = torch.randn(n, k, generator=g)
+        params = make_params(kernel_type, ())
+        s = torch.tensor(start, dtype=torch.int32)
+        e = torch.tensor(end, dtype=torch.int32)
+        args = tuple(t.to(device) for t in (x1, x2, rhs, params, s, e))
+        defines = MatmulSingleConfiguration(kernel_type).make_config(args)
+        defines["MATMUL_VARIANT"] = variant
+        result = load_native("matmul", defines).call(*args)
+        f = lambda t: t.detach().cpu().numpy()
+        expected = oracle.matmul(kernel_type, *(f(t) for t in args))
+        assert_close(result, expected)
+        for blk, (lo, hi) in enumerate(zip(start, end)):
+            if lo >= hi:
+                assert torch.all(result[blk * 128:(blk + 1) * 128] == 0)
+
+
+@pytest.mark.parametrize("kernel_type", ["rbf", "spectral", "locally_periodic"])
+def test_param_grad_degenerate_ranges(kernel_type):
+    """Same degenerate patterns for the parameter gradient (matmul_bwd)."""
+    from tests.conftest import make_params
+
+    g = torch.Generator().manual_seed(6)
+    device = torch.device("cuda:0")
+    for m, n, k, start, end in [
+        (300, 300, 3, [0, 120, 290], [50, 120, 400]),
+        (300, 300, 8, [10, 10, 10], [10, 10, 10]),
+        (1, 1, 1, [0], [1]),
+        (5, 700, 17, [3], [699]),
+    ]:
+        x1 = torch.sort(torch.rand(m, generator=g) * 10)[0]
+        x2 = torch.sort(torch.rand(n, generator=g) * 10)[0]
+        rhs = torch.randn(n, k, generator=g)
+        out_grad = torch.randn(m, k, generator=g)
+        out_grad = out_grad / torch.linalg.norm(out_grad)  # as in test_matmul_bwd
+        params = make_params(kernel_type, ())
+        s = torch.tensor(start, dtype=torch.int32)
+        e = torch.tensor(end, dtype=torch.int32)
+        args = tuple(t.to(device) for t in (x1, x2, rhs, params, s, e, out_grad))
+        defines = MatmulBwdConfiguration(kernel_type).make_config(args)
+        result = load_native("matmul_bwd", defines).call(*args)
+        f = lambda t: t.detach().cpu().numpy()
+        expected = oracle.param_grad(kernel_type, f(x1), f(x2), f(out_grad), f(rhs), f(params), f(s), f(e))
+        err = np.abs(result.cpu().double().numpy() - expected)
+        assert np.all(err <= _grad_tolerance(expected)), (result.cpu().numpy(), expected)
