@@ -187,3 +187,29 @@ def test_ranges_at_full_size_bit_exact():
         s_o, e_o = oracle_ranges.make_ranges(h["cutoff"], h["x"], x2.numpy(), align=align)
         np.testing.assert_array_equal(s_dev.cpu().numpy(), s_o)
         np.testing.assert_array_equal(e_dev.cpu().numpy(), e_o)
+
+
+def test_c1_dense_check():
+    """BASELINE config 1 (the reference's CPU-runnable case): rbf, n = 4096, k = 1, l = sigma = 1,
+    cutoff 8, checked against the full dense float64 product on the CPU."""
+    n = 4096
+    g = torch.Generator().manual_seed(1001)
+    x = torch.sort(torch.rand(n, generator=g) * 100.0)[0]
+    rhs = torch.randn(n, 1, generator=g)
+    params = torch.tensor([1.0, 1.0])
+    device = torch.device("cuda:0")
+    xd = x.to(device)
+    start, end = make_ranges(8.0, xd)
+    args = (xd, xd, rhs.to(device), params.to(device), start, end)
+    for variant in (None, "block", "mfma_f32", "valu"):
+        defines = MatmulSingleConfiguration("rbf").make_config(args)
+        if variant:
+            defines["MATMUL_VARIANT"] = variant
+        out = load_native("matmul", defines).call(*args)
+        expected = oracle.matmul("rbf", x.numpy(), x.numpy(), rhs.numpy(), params.numpy(),
+                                 start.cpu().numpy(), end.cpu().numpy())
+        err = np.abs(out.cpu().double().numpy() - expected)
+        assert np.all(err <= 1e-5 + 1e-4 * np.abs(expected)), (variant, err.max())
+        # cutoff 8 l: what the band leaves out is below exp(-32) per entry
+        dense = oracle.kernel_matrix("rbf", x.numpy(), x.numpy(), params.numpy()) @ rhs.double().numpy()
+        assert np.abs(out.cpu().double().numpy() - dense).max() < 2e-5
