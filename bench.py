@@ -41,7 +41,7 @@ WORKLOADS = {
 }
 
 # (FETCH_SIZE 3543.6 KiB x 2.00 + WRITE_SIZE 50000.0 KiB x 1.00) x 1024
-MEASURED_TRAFFIC_BYTES = {"headline": 58668032}
+MEASURED_TRAFFIC_BYTES = {"headline": 58665574}
 
 FLOPS_PER_PAIR = {"rbf": lambda k: 5 + 2 * k, "spectral": lambda k: 8 + 2 * k,
                   "locally_periodic": lambda k: 10 + 2 * k}
@@ -181,17 +181,21 @@ def main() -> int:
     achieved_tflops = pairs * flops_per_pair / (kernel_ms_avg * 1e-3) / 1e12
 
     # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
-    # profiles/fwd_spectral_f16_headline_counters.md (only measured for the default headline run).
+    # profiles/fwd_table_f16_headline_counters.md (only measured for the default headline run).
     traffic = None
     if args.workload == "headline" and args.batch is None and args.variant in ("auto", "mfma_f16"):
         traffic = MEASURED_TRAFFIC_BYTES["headline"]
 
-    # Kernel the launch table picks for this workload / variant (phase-split only for spectral
-    # kernels with at most 16 rhs columns).
-    phase_split = w["kernel"] == "spectral" and k <= 16
+    # Kernel the launch table picks for this workload / variant: column tables (spectral in
+    # phase-split form) for rbf / spectral with at most 16 rhs columns, the shared-operand kernel
+    # for large rbf / locally periodic problems, direct evaluation otherwise.
+    row_block_items = ((n + 127) // 128) * max(batch, 1)
+    table = w["kernel"] in ("spectral", "rbf") and k <= 16
+    shared = w["kernel"] != "spectral" and k <= 16 and row_block_items >= 4096
+    auto_kernel = "km::fwd_block" if shared else ("km::fwd_table_f16" if table else "km::fwd_mfma_f16")
     kernel_name = "km::param_grad_partial" if is_grad else {
-        "auto": "km::fwd_spectral_f16" if phase_split else "km::fwd_mfma_f16",
-        "mfma_f16": "km::fwd_spectral_f16" if phase_split else "km::fwd_mfma_f16",
+        "auto": auto_kernel,
+        "mfma_f16": "km::fwd_table_f16" if table else "km::fwd_mfma_f16",
         "mfma_f16_direct": "km::fwd_mfma_f16", "block": "km::fwd_block",
         "mfma_f32": "km::fwd_mfma_f32", "valu": "km::fwd_valu"}[args.variant]
 

@@ -82,12 +82,23 @@ static int check_common(const char* op, int kernel_type, int batch_rank, const i
 // (measured: 1024 beats 2048 and 4096 from 157 to 3128 row-block items).
 // ---------------------------------------------------------------------------------------
 static const long long TARGET_WAVES = 1024;
+// Row-block items from which the workgroup-shared forward kernel is considered.
+static const long long BLOCK_VARIANT_MIN_ITEMS = 4096;
 
 static int make_plan(const MatmulProblem& p, const km_launch_options* opt, MatmulPlan* plan) {
     int variant = opt ? opt->variant : KM_VARIANT_AUTO;
     plan->phase_split = 0;
     if (variant == KM_VARIANT_AUTO) {
-        variant = KM_VARIANT_MFMA_F16;
+        // Measured on gfx950 (n = 1e5 ... 1e6, batch 2 ... 8): with up to 16 rhs columns and enough
+        // row blocks to fill the device several times, sharing the rhs operand between four row
+        // blocks wins for the rbf (7 %) and locally periodic (12-18 %) kernels; the phase-split
+        // spectral kernel and everything with wider rhs or fewer row blocks is faster with one
+        // wavefront per row block.
+        const long long row_blocks = (p.m + KM_BLOCK_SIZE - 1) / KM_BLOCK_SIZE;
+        const bool shared = p.kernel_type != KM_KERNEL_SPECTRAL && p.k <= 16 &&
+                            row_blocks * p.num_batches >= BLOCK_VARIANT_MIN_ITEMS &&
+                            !(opt && (opt->rows_per_wave != 0 || opt->col_splits > 1));
+        variant = shared ? KM_VARIANT_BLOCK : KM_VARIANT_MFMA_F16;
     }
     if (variant != KM_VARIANT_VALU && variant != KM_VARIANT_MFMA_F32 && variant != KM_VARIANT_MFMA_F16 &&
         variant != KM_VARIANT_MFMA_F16_DIRECT && variant != KM_VARIANT_BLOCK) {
@@ -114,11 +125,13 @@ static int make_plan(const MatmulProblem& p, const km_launch_options* opt, Matmu
         plan->tail_balance = 0;
         return KM_OK;
     }
-    // The phase-split spectral kernel keeps two accumulator sets per rhs column group, so it
-    // takes at most 32 rhs columns per pass.
-    const bool phase_split = variant == KM_VARIANT_MFMA_F16 && p.kernel_type == KM_KERNEL_SPECTRAL && p.k <= 16;
-    if (variant == KM_VARIANT_MFMA_F16 && !phase_split) {
-        // Only spectral kernels with up to 16 rhs columns gain from the phase-split form.
+    // Table kernel (column tables in LDS, folded coordinates): rbf and spectral kernels with up
+    // to 16 rhs columns; the spectral one in phase-split form, which keeps two accumulator sets
+    // per rhs column group.  Everything else evaluates directly.
+    const bool table = variant == KM_VARIANT_MFMA_F16 && p.k <= 16 &&
+                       (p.kernel_type == KM_KERNEL_SPECTRAL || p.kernel_type == KM_KERNEL_RBF);
+    const bool phase_split = table && p.kernel_type == KM_KERNEL_SPECTRAL;
+    if (variant == KM_VARIANT_MFMA_F16 && !table) {
         variant = KM_VARIANT_MFMA_F16_DIRECT;
         plan->variant = variant;
     }
@@ -160,8 +173,8 @@ static int make_plan(const MatmulProblem& p, const km_launch_options* opt, Matmu
         }
     }
     // LDS per workgroup must stay within 64 KiB: the cross-wavefront reduction buffer takes
-    // S * R * G KiB and the phase-split kernel's tables 8.1 KiB per wavefront.
-    while (S > 1 && S * (R * G + (phase_split ? 9 : 0)) > 64) {
+    // S * R * G KiB and the table kernel's tables 8.1 KiB per wavefront.
+    while (S > 1 && S * (R * G + (table ? 9 : 0)) > 64) {
         S /= 2;
     }
     plan->row_groups = R;

@@ -660,11 +660,13 @@ __device__ __forceinline__ void rhs_load(const FwdArgs& a, const WaveView& w, in
     }
 }
 
-template <int G, int R>
-__device__ __forceinline__ void fwd_spectral_f16_body(const FwdArgs& a, float* lds, const WaveView& w,
-                                                      int row0) {
-    constexpr int KT = KM_KERNEL_SPECTRAL;
-    constexpr int GE = 2 * G;  // accumulator groups: [cos part of g = 0..G) , sin part of g = 0..G)]
+template <int KT, int G, int R>
+__device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds, const WaveView& w,
+                                                   int row0) {
+    static_assert(KT == KM_KERNEL_SPECTRAL || KT == KM_KERNEL_RBF, "table kernel: rbf or spectral");
+    constexpr bool PHASE = KT == KM_KERNEL_SPECTRAL;
+    // Accumulator groups; phase-split: [cos part of g = 0..G), sin part of g = 0..G)].
+    constexpr int GE = PHASE ? 2 * G : G;
     constexpr int CH = KM_PHASE_CHUNK;
 
     const int lane = threadIdx.x & 63;
@@ -703,7 +705,7 @@ __device__ __forceinline__ void fwd_spectral_f16_body(const FwdArgs& a, float* l
         const int c = kbase + 16 * g + li;
         rhs_lane[g] = (unsigned)(8 * kk * a.rhs_s0 + min(c, a.k - 1) * a.rhs_s1);
 #pragma unroll
-        for (int part = 0; part < 2; part++) {
+        for (int part = 0; part < GE / G; part++) {
             colmask[part * G + g] = c < a.k;
             shift[part * G + g] = 100;
             scale[part * G + g] = c < a.k ? __builtin_ldexpf(1.0f, 100) : 0.0f;
@@ -766,10 +768,12 @@ __device__ __forceinline__ void fwd_spectral_f16_body(const FwdArgs& a, float* l
             const float bb = xd - xv;
             const float err = (xv - (xd - bb)) - (ref + bb);  // exact rounding error of xd
             const float xs = xd * kc.s;
-            const float th = phase_rev(kc.f, xv, c_ref);
             tab_x2[q] = xv;
-            tab_cos[q] = __builtin_amdgcn_cosf(th);
-            tab_sin[q] = __builtin_amdgcn_sinf(th);
+            if (PHASE) {
+                const float th = phase_rev(kc.f, xv, c_ref);
+                tab_cos[q] = __builtin_amdgcn_cosf(th);
+                tab_sin[q] = __builtin_amdgcn_sinf(th);
+            }
             tab_xs[q] = xs;
             if ((q & 31) == 0) {
                 tab_ref[q >> 5] = ref;
@@ -800,13 +804,18 @@ __device__ __forceinline__ void fwd_spectral_f16_body(const FwdArgs& a, float* l
 #pragma unroll
                 for (int t = 0; t < 8; t += 4) {
                     const float4v vx = *(const float4v*)((FOLD ? tab_xs : tab_x2) + off + t);
-                    const float4v vc = *(const float4v*)(tab_cos + off + t);
-                    const float4v vs = *(const float4v*)(tab_sin + off + t);
 #pragma unroll
                     for (int u = 0; u < 4; u++) {
                         x2v[t + u] = vx[u];
-                        cb[t + u] = vc[u];
-                        sb[t + u] = vs[u];
+                    }
+                    if (PHASE) {
+                        const float4v vc = *(const float4v*)(tab_cos + off + t);
+                        const float4v vs = *(const float4v*)(tab_sin + off + t);
+#pragma unroll
+                        for (int u = 0; u < 4; u++) {
+                            cb[t + u] = vc[u];
+                            sb[t + u] = vs[u];
+                        }
                     }
                 }
                 const float ref = FOLD ? tab_ref[(c0 - chunk0) >> 5] : 0.0f;
@@ -815,8 +824,12 @@ __device__ __forceinline__ void fwd_spectral_f16_body(const FwdArgs& a, float* l
                 for (int g = 0; g < G; g++) {
 #pragma unroll
                     for (int t = 0; t < 8; t++) {
-                        braw[g][t] = raw[g][t] * cb[t];
-                        braw[G + g][t] = raw[g][t] * sb[t];
+                        if (PHASE) {
+                            braw[g][t] = raw[g][t] * cb[t];
+                            braw[GE - G + g][t] = raw[g][t] * sb[t];
+                        } else {
+                            braw[g][t] = raw[g][t];
+                        }
                     }
                 }
                 f16_step<KM_KERNEL_RBF, GE, R, FOLD>(x2v, braw, x1v, kc, colmask, shift, scale, acc, ref);
@@ -834,34 +847,39 @@ __device__ __forceinline__ void fwd_spectral_f16_body(const FwdArgs& a, float* l
         __builtin_amdgcn_wave_barrier();
     }
 
-    // out = sigma * (cos A * P + sin A * Q) with the power-of-two scales undone; A for the rows
-    // this lane holds in the accumulator layout.
-    // cos A / sin A are formed once per row by the lane that holds the row's coordinate
-    // (x1v: row 16 r + lane % 16) and fetched across lanes into the accumulator layout
-    // (rows 16 r + 4 (lane / 16) + v).
+    // Power-of-two scales undone and sigma applied; phase-split:
+    // out = sigma * (cos A * P + sin A * Q), with cos A / sin A formed once per row by the lane
+    // that holds the row's coordinate (x1v: row 16 r + lane % 16) and fetched across lanes into
+    // the accumulator layout (rows 16 r + 4 (lane / 16) + v).
     float4v res[R][G];
 #pragma unroll
     for (int r = 0; r < R; r++) {
-        const float th = phase_rev(kc.f, x1v[r], c_ref);
-        const float ca_own = __builtin_amdgcn_cosf(th);
-        const float sa_own = __builtin_amdgcn_sinf(th);
         float ca[4], sa[4];
+        if (PHASE) {
+            const float th = phase_rev(kc.f, x1v[r], c_ref);
+            const float ca_own = __builtin_amdgcn_cosf(th);
+            const float sa_own = __builtin_amdgcn_sinf(th);
 #pragma unroll
-        for (int v = 0; v < 4; v++) {
-            ca[v] = __shfl(ca_own, 4 * kk + v, 64);
-            sa[v] = __shfl(sa_own, 4 * kk + v, 64);
+            for (int v = 0; v < 4; v++) {
+                ca[v] = __shfl(ca_own, 4 * kk + v, 64);
+                sa[v] = __shfl(sa_own, 4 * kk + v, 64);
+            }
         }
 #pragma unroll
         for (int g = 0; g < G; g++) {
             const float up = __builtin_ldexpf(sigma, -shift[g] - KM_F16_KSCALE_LOG2);
-            const float uq = __builtin_ldexpf(sigma, -shift[G + g] - KM_F16_KSCALE_LOG2);
+            const float uq = __builtin_ldexpf(sigma, -shift[GE - G + g] - KM_F16_KSCALE_LOG2);
 #pragma unroll
             for (int v = 0; v < 4; v++) {
-                res[r][g][v] = ca[v] * (acc[r][g][v] * up) + sa[v] * (acc[r][G + g][v] * uq);
+                if (PHASE) {
+                    res[r][g][v] = ca[v] * (acc[r][g][v] * up) + sa[v] * (acc[r][GE - G + g][v] * uq);
+                } else {
+                    res[r][g][v] = acc[r][g][v] * up;
+                }
             }
         }
-        // One row group at a time: keeps the double-precision phase arithmetic of several
-        // groups from being interleaved, which costs registers for nothing.
+        // One row group at a time keeps the phase arithmetic of several groups from being
+        // interleaved, which costs registers for nothing.
         __builtin_amdgcn_sched_barrier(0);
     }
     float* __restrict__ out = a.out + w.b * (long long)a.m * a.k;
@@ -872,8 +890,8 @@ __device__ __forceinline__ void fwd_spectral_f16_body(const FwdArgs& a, float* l
     }
 }
 
-template <int G, int R>
-__global__ void __launch_bounds__(512, 3) fwd_spectral_f16(const FwdArgs a) {
+template <int KT, int G, int R>
+__global__ void __launch_bounds__(512, 3) fwd_table_f16(const FwdArgs a) {
     extern __shared__ float lds[];
     KM_TL_BEGIN();
     const ItemRef it = decode_item(a);
@@ -884,13 +902,13 @@ __global__ void __launch_bounds__(512, 3) fwd_spectral_f16(const FwdArgs a) {
     if constexpr (R == 8) {
         if (it.small) {
             const WaveView w = wave_view(a, it.item, 1, &chunk_in_block);
-            fwd_spectral_f16_body<G, 1>(a, lds, w, w.row_block * KM_BLOCK_SIZE + 16 * it.piece);
+            fwd_table_f16_body<KT, G, 1>(a, lds, w, w.row_block * KM_BLOCK_SIZE + 16 * it.piece);
             KM_TL_END();
             return;
         }
     }
     const WaveView w = wave_view(a, it.item, a.chunks_per_block, &chunk_in_block);
-    fwd_spectral_f16_body<G, R>(a, lds, w, w.row_block * KM_BLOCK_SIZE + chunk_in_block * (16 * R));
+    fwd_table_f16_body<KT, G, R>(a, lds, w, w.row_block * KM_BLOCK_SIZE + chunk_in_block * (16 * R));
     KM_TL_END();
 }
 
@@ -961,16 +979,17 @@ template <int KT, int G, int R>
 static hipError_t launch_mfma(const FwdArgs& a, int variant, int S, unsigned gx, unsigned gy,
                               hipStream_t stream) {
     const size_t lds = S > 1 ? (size_t)S * R * G * 4 * 64 * sizeof(float) : 0;
-    if (variant == KM_VARIANT_MFMA_F16 && KT == KM_KERNEL_SPECTRAL) {
-        // Instantiated only for the shapes the launch table can pick (register budget).
-        if constexpr (G == 1) {
+    constexpr bool HAS_TABLE_KERNEL = (KT == KM_KERNEL_SPECTRAL || KT == KM_KERNEL_RBF) && G == 1;
+    if (variant == KM_VARIANT_MFMA_F16) {
+        // The table kernel exists for the shapes the launch table can pick (register budget).
+        if constexpr (HAS_TABLE_KERNEL) {
             const size_t table = (size_t)S * KM_PHASE_TABLE_FLOATS * sizeof(float);
-            hipLaunchKernelGGL((fwd_spectral_f16<G, R>), dim3(gx, gy, 1),
-                               dim3(64 * S, 1, 1), table + lds, stream, a);
+            hipLaunchKernelGGL((fwd_table_f16<KT, G, R>), dim3(gx, gy, 1), dim3(64 * S, 1, 1), table + lds,
+                               stream, a);
         } else {
             return hipErrorInvalidConfiguration;
         }
-    } else if (variant == KM_VARIANT_MFMA_F16 || variant == KM_VARIANT_MFMA_F16_DIRECT) {
+    } else if (variant == KM_VARIANT_MFMA_F16_DIRECT) {
         // Wide rhs tiles with many row groups exceed the register file; the launch table never
         // picks them.
         if constexpr (G * R <= 8) {
