@@ -305,10 +305,13 @@ def test_matmul_degenerate_ranges(kernel_type, variant):
         (1, 1, 1, [0], [1]),
         (129, 1, 2, [0, 0], [128, 1]),
         (5, 700, 17, [3], [699]),
+        # ranges that jump back and forth between neighbouring row blocks, with gaps
+        (1000, 1200, 16, [900, 0, 600, 610, 100, 1190, 300, 0], [1200, 40, 900, 611, 500, 1200, 301, 1200]),
     ]:
         x1 = torch.sort(torch.rand(m, generator=g) * 10)[0]
         x2 = torch.sort(torch.rand(n, generator=g) * 10)[0]
         rhs = torch.randn(n, k, generator=g)
+        rhs = rhs / torch.linalg.norm(rhs, dim=-2, keepdim=True)  # as the example data does
         params = make_params(kernel_type, ())
         s = torch.tensor(start, dtype=torch.int32)
         e = torch.tensor(end, dtype=torch.int32)
