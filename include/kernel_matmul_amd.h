@@ -53,11 +53,14 @@ extern "C" {
  * only select among ahead-of-time instantiated kernels. */
 typedef struct km_launch_options {
     int variant;          /* 0 = table, 1 = VALU FMA contraction, 2 = fp32 MFMA contraction,
-                             3 = split-fp16 (hi+lo) MFMA contraction with fp32 accumulation
-                             (spectral kernels in phase-split form), 4 = the same with the
-                             cosine evaluated per pair, 5 = split-fp16 MFMA with the rhs operand
-                             prepared once per workgroup of four row blocks (the table's choice
-                             for large problems; rows_per_wave / col_splits must stay 0) */
+                             3 = split-fp16 (hi+lo) MFMA contraction with fp32 accumulation; rbf
+                             and spectral kernels with at most 16 rhs columns go through
+                             per-wavefront column tables (spectral in phase-split form),
+                             4 = split-fp16 MFMA with the kernel evaluated directly per pair,
+                             5 = split-fp16 MFMA with the rhs operand prepared once per workgroup
+                             of four row blocks (rows_per_wave / col_splits must stay 0).
+                             The table picks 5 for large rbf / locally periodic problems with at
+                             most 16 rhs columns and 3 otherwise. */
     int rows_per_wave;    /* 0 = table; else 16, 32, 64 or 128 rows of x1 per wavefront */
     int col_splits;       /* 0 = table; else 1, 2, 4 or 8 wavefronts sharing one row range */
     int reserved;
