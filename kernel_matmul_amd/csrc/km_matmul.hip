@@ -430,12 +430,17 @@ __device__ __forceinline__ void f16_load(const FwdArgs& a, const WaveView& w, in
 // One step of 32 columns: convert this lane's 8 rhs values per column group to hi/lo halves
 // (rescaling the accumulators first if a value would leave the fp16 range), then for every
 // row group evaluate 8 kernel entries, split them and issue the three MFMAs.
-template <int KT, int G, int R, bool FOLD = false>
+// PARTS = 2 (phase-split form): every rhs value enters twice, multiplied by cb[] and by sb[]
+// (|cb|, |sb| <= 1), into the accumulator groups g and G + g; both share the column's scale,
+// which is taken from |rhs| alone.
+template <int KT, int G, int R, bool FOLD = false, int PARTS = 1>
 __device__ __forceinline__ void f16_step(const float (&x2v)[8], const float (&raw)[G][8],
                                          const float (&x1v)[R], const KernelConsts& kc,
                                          const bool (&colmask)[G], int (&shift)[G],
-                                         float (&scale)[G], float4v (&acc)[R][G], float ref = 0.0f) {
-    half8v bhi[G], blo[G];
+                                         float (&scale)[G], float4v (&acc)[R][G * PARTS], float ref = 0.0f,
+                                         const float* cb = nullptr, const float* sb = nullptr) {
+    constexpr int GE = G * PARTS;
+    half8v bhi[GE], blo[GE];
 #pragma unroll
     for (int g = 0; g < G; g++) {
         // Largest magnitude of this rhs column over the step's 32 columns (the 4 lanes that
@@ -456,7 +461,10 @@ __device__ __forceinline__ void f16_step(const float (&x2v)[8], const float (&ra
                 const float factor = __builtin_ldexpf(1.0f, new_shift - shift[g]);
 #pragma unroll
                 for (int r = 0; r < R; r++) {
-                    acc[r][g] *= factor;
+#pragma unroll
+                    for (int part = 0; part < PARTS; part++) {
+                        acc[r][part * G + g] *= factor;
+                    }
                 }
                 shift[g] = new_shift;
                 scale[g] = __builtin_ldexpf(1.0f, new_shift);
@@ -467,7 +475,18 @@ __device__ __forceinline__ void f16_step(const float (&x2v)[8], const float (&ra
         for (int t = 0; t < 8; t++) {
             rv[t] = raw[g][t] * scale[g];
         }
-        split_f16x8(rv, kc.one, &bhi[g], &blo[g]);
+        if (PARTS == 2) {
+            float vc[8], vs[8];
+#pragma unroll
+            for (int t = 0; t < 8; t++) {
+                vc[t] = rv[t] * cb[t];
+                vs[t] = rv[t] * sb[t];
+            }
+            split_f16x8(vc, kc.one, &bhi[g], &blo[g]);
+            split_f16x8(vs, kc.one, &bhi[G + g], &blo[G + g]);
+        } else {
+            split_f16x8(rv, kc.one, &bhi[g], &blo[g]);
+        }
     }
 
 #pragma unroll
@@ -481,7 +500,7 @@ __device__ __forceinline__ void f16_step(const float (&x2v)[8], const float (&ra
         const half8v ahi = join_half2x4(h2);
         const half8v alo = join_half2x4(l2);
 #pragma unroll
-        for (int g = 0; g < G; g++) {
+        for (int g = 0; g < GE; g++) {
             acc[r][g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahi, bhi[g], acc[r][g], 0, 0, 0);
             acc[r][g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahi, blo[g], acc[r][g], 0, 0, 0);
             acc[r][g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(alo, bhi[g], acc[r][g], 0, 0, 0);
@@ -696,20 +715,17 @@ __device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds,
         x1v[r] = w.x1[(long long)row * a.x1_s];
     }
 
-    bool colmask[GE];
+    bool colmask[G];
     unsigned rhs_lane[G];
-    int shift[GE];
-    float scale[GE];
+    int shift[G];
+    float scale[G];
 #pragma unroll
     for (int g = 0; g < G; g++) {
         const int c = kbase + 16 * g + li;
         rhs_lane[g] = (unsigned)(8 * kk * a.rhs_s0 + min(c, a.k - 1) * a.rhs_s1);
-#pragma unroll
-        for (int part = 0; part < GE / G; part++) {
-            colmask[part * G + g] = c < a.k;
-            shift[part * G + g] = 100;
-            scale[part * G + g] = c < a.k ? __builtin_ldexpf(1.0f, 100) : 0.0f;
-        }
+        colmask[g] = c < a.k;
+        shift[g] = 100;
+        scale[g] = c < a.k ? __builtin_ldexpf(1.0f, 100) : 0.0f;
     }
 
     float4v acc[R][GE];
@@ -819,20 +835,7 @@ __device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds,
                     }
                 }
                 const float ref = FOLD ? tab_ref[(c0 - chunk0) >> 5] : 0.0f;
-                float braw[GE][8];
-#pragma unroll
-                for (int g = 0; g < G; g++) {
-#pragma unroll
-                    for (int t = 0; t < 8; t++) {
-                        if (PHASE) {
-                            braw[g][t] = raw[g][t] * cb[t];
-                            braw[GE - G + g][t] = raw[g][t] * sb[t];
-                        } else {
-                            braw[g][t] = raw[g][t];
-                        }
-                    }
-                }
-                f16_step<KM_KERNEL_RBF, GE, R, FOLD>(x2v, braw, x1v, kc, colmask, shift, scale, acc, ref);
+                f16_step<KM_KERNEL_RBF, G, R, FOLD, GE / G>(x2v, raw, x1v, kc, colmask, shift, scale, acc, ref, cb, sb);
                 if (c0 + 32 < chunk_end) {
                     rhs_load<G>(a, w, c0 + 32, chunk_end, kk, rhs_lane, raw);
                 }
@@ -868,11 +871,10 @@ __device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds,
 #pragma unroll
         for (int g = 0; g < G; g++) {
             const float up = __builtin_ldexpf(sigma, -shift[g] - KM_F16_KSCALE_LOG2);
-            const float uq = __builtin_ldexpf(sigma, -shift[GE - G + g] - KM_F16_KSCALE_LOG2);
 #pragma unroll
             for (int v = 0; v < 4; v++) {
                 if (PHASE) {
-                    res[r][g][v] = ca[v] * (acc[r][g][v] * up) + sa[v] * (acc[r][GE - G + g][v] * uq);
+                    res[r][g][v] = ca[v] * (acc[r][g][v] * up) + sa[v] * (acc[r][GE - G + g][v] * up);
                 } else {
                     res[r][g][v] = acc[r][g][v] * up;
                 }
