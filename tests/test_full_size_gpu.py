@@ -1,4 +1,4 @@
-"""Parity at the full BASELINE.json sizes through properties that do not need a dense oracle:
+"""Parity at the full sizes of the benchmark configurations through properties that do not need a dense oracle:
 oracle on sampled row blocks, linearity in rhs, symmetry of the bilinear form, agreement of the
 three contraction variants, d/d(outputscale) identity, index lookups against per-entry closed
 forms, and bit-exact device ranges at n = 10^6."""
@@ -190,7 +190,7 @@ def test_ranges_at_full_size_bit_exact():
 
 
 def test_c1_dense_check():
-    """BASELINE config 1 (the reference's CPU-runnable case): rbf, n = 4096, k = 1, l = sigma = 1,
+    """Benchmark configuration 1 (the reference's CPU-runnable case): rbf, n = 4096, k = 1, l = sigma = 1,
     cutoff 8, checked against the full dense float64 product on the CPU."""
     n = 4096
     g = torch.Generator().manual_seed(1001)
