@@ -125,10 +125,9 @@ def load_library():
 
 
 def _raise(lib, status: int):
-    message = lib.km_last_error().decode("utf-8", "replace")
-    if status == -1:
-        raise ValueError(message)
-    raise RuntimeError(message)
+    # Every failed check of the reference's entry points is a TORCH_CHECK, i.e. a RuntimeError
+    # (native/common/entrypoint.h:3-14).
+    raise RuntimeError(lib.km_last_error().decode("utf-8", "replace"))
 
 
 def _i64(values: Sequence[int]):
@@ -144,7 +143,55 @@ def _tensor_args(t: Tensor):
 
 
 def _stream(device: torch.device):
-    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+    index = device.index
+    if index is None:
+        index = torch.cuda.current_device()
+    return ctypes.c_void_p(torch._C._cuda_getCurrentRawStream(index))
+
+
+class _on_device:
+    """Makes ``device`` current for the launch; costs nothing when it already is."""
+
+    __slots__ = ("_guard",)
+
+    def __init__(self, device: torch.device):
+        index = device.index
+        self._guard = None
+        if index is not None and index != torch.cuda.current_device():
+            self._guard = torch.cuda.device(index)
+
+    def __enter__(self):
+        if self._guard is not None:
+            self._guard.__enter__()
+
+    def __exit__(self, *exc):
+        if self._guard is not None:
+            return self._guard.__exit__(*exc)
+        return False
+
+
+# Validated calls, keyed by everything the validation looked at (shapes, strides, dtypes,
+# devices).  A repeated call with the same signature skips the checks and reuses the ctypes
+# stride / size arrays: only the data pointers, the output and the stream are new.
+_PREPARED: dict = {}
+_PREPARED_LIMIT = 512
+
+
+def _signature(op: str, kernel_type: str, tensors) -> tuple:
+    key = [op, kernel_type]
+    for t in tensors:
+        key.append(t.shape)
+        key.append(t.stride())
+        key.append(t.dtype)
+        key.append(t.device)
+    return tuple(key)
+
+
+def _remember(key, value):
+    if len(_PREPARED) >= _PREPARED_LIMIT:
+        _PREPARED.clear()
+    _PREPARED[key] = value
+    return value
 
 
 # -- the checks of the reference's entry points (native/common/entrypoint.h:3-14) ----------
@@ -211,60 +258,95 @@ def _check_matrix_inputs(kernel_type, x1, x2, params, start, end):
 
 
 def matmul(kernel_type: str, x1: Tensor, x2: Tensor, rhs: Tensor, params: Tensor, start: Tensor,
-           end: Tensor, options: LaunchOptions | None = None) -> Tensor:
-    """out[..., m, k] = K(x1, x2)[mask] @ rhs   (C ABI: km_matmul)."""
-    kid = _kernel_id(kernel_type)
-    check_cuda(rhs)
-    check_float(rhs)
-    batch_shape = _check_matrix_inputs(kernel_type, x1, x2, params, start, end)
-    _check_batch("rhs", rhs, batch_shape, 2)
-    m, n, k = x1.shape[-1], x2.shape[-1], rhs.shape[-1]
-    if rhs.shape[-2] != n:
-        raise RuntimeError(f"rhs has {rhs.shape[-2]} rows, x2 has {n} points")
-    lib = load_library()
-    out = torch.empty((*batch_shape, m, k), dtype=torch.float32, device=x1.device)
-    with torch.cuda.device(x1.device):
-        status = lib.km_matmul(
-            kid, len(batch_shape), _i64(batch_shape), m, n, k,
-            *_tensor_args(x1), *_tensor_args(x2), *_tensor_args(rhs), *_tensor_args(params),
-            *_tensor_args(start), *_tensor_args(end), _ptr(out),
-            ctypes.byref(options) if options is not None else None, _stream(x1.device),
-        )
+           end: Tensor, options: LaunchOptions | None = None, out: Tensor | None = None) -> Tensor:
+    """out[..., m, k] = K(x1, x2)[mask] @ rhs   (C ABI: km_matmul).
+
+    ``out`` (optional) is a contiguous fp32 tensor of the result's shape to write into."""
+    tensors = (x1, x2, rhs, params, start, end)
+    key = _signature("matmul", kernel_type, tensors)
+    prepared = _PREPARED.get(key)
+    if prepared is None:
+        kid = _kernel_id(kernel_type)
+        check_cuda(rhs)
+        check_float(rhs)
+        batch_shape = _check_matrix_inputs(kernel_type, x1, x2, params, start, end)
+        _check_batch("rhs", rhs, batch_shape, 2)
+        m, n, k = x1.shape[-1], x2.shape[-1], rhs.shape[-1]
+        if rhs.shape[-2] != n:
+            raise RuntimeError(f"rhs has {rhs.shape[-2]} rows, x2 has {n} points")
+        prepared = _remember(key, (
+            load_library().km_matmul, (kid, len(batch_shape), _i64(batch_shape), m, n, k),
+            tuple(_i64(t.stride()) for t in tensors), tuple(t.numel() > 0 for t in tensors),
+            (*batch_shape, m, k),
+        ))
+    fn, head, strides, nonempty, out_shape = prepared
+    device = x1.device
+    if out is None:
+        out = torch.empty(out_shape, dtype=torch.float32, device=device)
+    elif (tuple(out.shape) != out_shape or out.dtype != torch.float32 or out.device != device
+          or not out.is_contiguous()):
+        raise RuntimeError(f"out must be a contiguous float32 tensor of shape {out_shape} on {device}")
+    call_args = []
+    for t, st, filled in zip(tensors, strides, nonempty):
+        call_args.append(t.data_ptr() if filled else None)
+        call_args.append(st)
+    with _on_device(device):
+        status = fn(*head, *call_args, out.data_ptr() if out.numel() > 0 else None,
+                    ctypes.byref(options) if options is not None else None, _stream(device))
     if status != 0:
-        _raise(lib, status)
+        _raise(load_library(), status)
     return out
 
 
 def param_grad(kernel_type: str, x1: Tensor, x2: Tensor, left: Tensor, right: Tensor,
-               params: Tensor, start: Tensor, end: Tensor) -> Tensor:
-    """grad[..., P] of sum((left @ right^T) * K[mask]) w.r.t. params   (C ABI: km_param_grad)."""
-    kid = _kernel_id(kernel_type)
-    for t in (left, right):
-        check_cuda(t)
-        check_float(t)
-    batch_shape = _check_matrix_inputs(kernel_type, x1, x2, params, start, end)
-    _check_batch("left", left, batch_shape, 2)
-    _check_batch("right", right, batch_shape, 2)
-    m, n, c = x1.shape[-1], x2.shape[-1], left.shape[-1]
-    if left.shape[-2] != m or right.shape[-2] != n or right.shape[-1] != c:
-        raise RuntimeError(
-            f"left {tuple(left.shape)} / right {tuple(right.shape)} do not match a {m} x {n} matrix"
-        )
+               params: Tensor, start: Tensor, end: Tensor, out: Tensor | None = None) -> Tensor:
+    """grad[..., P] of sum((left @ right^T) * K[mask]) w.r.t. params   (C ABI: km_param_grad).
+
+    ``out`` (optional) is a contiguous fp32 tensor [..., P] to write into."""
+    tensors = (x1, x2, left, right, params, start, end)
+    key = _signature("param_grad", kernel_type, tensors)
+    prepared = _PREPARED.get(key)
+    if prepared is None:
+        kid = _kernel_id(kernel_type)
+        for t in (left, right):
+            check_cuda(t)
+            check_float(t)
+        batch_shape = _check_matrix_inputs(kernel_type, x1, x2, params, start, end)
+        _check_batch("left", left, batch_shape, 2)
+        _check_batch("right", right, batch_shape, 2)
+        m, n, c = x1.shape[-1], x2.shape[-1], left.shape[-1]
+        if left.shape[-2] != m or right.shape[-2] != n or right.shape[-1] != c:
+            raise RuntimeError(
+                f"left {tuple(left.shape)} / right {tuple(right.shape)} do not match a {m} x {n} matrix"
+            )
+        lib = load_library()
+        sizes = _i64(batch_shape)
+        need = lib.km_param_grad_workspace_size(kid, len(batch_shape), sizes, m, n, c)
+        prepared = _remember(key, (
+            (kid, len(batch_shape), sizes, m, n, c),
+            tuple(_i64(t.stride()) for t in tensors), tuple(t.numel() > 0 for t in tensors),
+            (*batch_shape, params.shape[-1]), need,
+        ))
+    head, strides, nonempty, out_shape, need = prepared
     lib = load_library()
-    grad = torch.empty((*batch_shape, params.shape[-1]), dtype=torch.float32, device=x1.device)
-    sizes = _i64(batch_shape)
-    need = lib.km_param_grad_workspace_size(kid, len(batch_shape), sizes, m, n, c)
-    workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=x1.device)
-    with torch.cuda.device(x1.device):
-        status = lib.km_param_grad(
-            kid, len(batch_shape), sizes, m, n, c,
-            *_tensor_args(x1), *_tensor_args(x2), *_tensor_args(left), *_tensor_args(right),
-            *_tensor_args(params), *_tensor_args(start), *_tensor_args(end),
-            _ptr(grad), ctypes.c_void_p(workspace.data_ptr()), need, _stream(x1.device),
-        )
+    device = x1.device
+    if out is None:
+        out = torch.empty(out_shape, dtype=torch.float32, device=device)
+    elif (tuple(out.shape) != out_shape or out.dtype != torch.float32 or out.device != device
+          or not out.is_contiguous()):
+        raise RuntimeError(f"out must be a contiguous float32 tensor of shape {out_shape} on {device}")
+    call_args = []
+    for t, st, filled in zip(tensors, strides, nonempty):
+        call_args.append(t.data_ptr() if filled else None)
+        call_args.append(st)
+    out_ptr = out.data_ptr() if out.numel() > 0 else None
+    workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=device)
+    with _on_device(device):
+        status = lib.km_param_grad(*head, *call_args, out_ptr, workspace.data_ptr(), need,
+                                   _stream(device))
     if status != 0:
         _raise(lib, status)
-    return grad
+    return out
 
 
 def index(kernel_type: str, x1: Tensor, x2: Tensor, params: Tensor, start: Tensor, end: Tensor,
@@ -294,7 +376,7 @@ def index(kernel_type: str, x1: Tensor, x2: Tensor, params: Tensor, start: Tenso
     out = torch.empty(shape, dtype=torch.float32, device=x1.device)
     rank = len(batch_shape)
     bi_ptrs, bi_strides, _keep = _batch_index_args(batch_indices, rank)
-    with torch.cuda.device(x1.device):
+    with _on_device(x1.device):
         status = lib.km_index(
             kid, rank, _i64(batch_shape), x1.shape[-1], x2.shape[-1],
             *_tensor_args(x1), *_tensor_args(x2), *_tensor_args(params),
@@ -343,7 +425,7 @@ def index_bwd(kernel_type: str, x1: Tensor, x2: Tensor, params: Tensor, start: T
     need = lib.km_index_bwd_workspace_size(row_index.numel())
     workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=x1.device)
     bi_ptrs, bi_strides, _keep = _batch_index_args(batch_indices, rank)
-    with torch.cuda.device(x1.device):
+    with _on_device(x1.device):
         status = lib.km_index_bwd(
             kid, rank, _i64(batch_shape), x1.shape[-1], x2.shape[-1],
             *_tensor_args(x1), *_tensor_args(x2), *_tensor_args(params),
@@ -364,7 +446,7 @@ def dense(kernel_type: str, x1: Tensor, x2: Tensor, params: Tensor, start: Tenso
     batch_shape = _check_matrix_inputs(kernel_type, x1, x2, params, start, end)
     lib = load_library()
     out = torch.empty((*batch_shape, x1.shape[-1], x2.shape[-1]), dtype=torch.float32, device=x1.device)
-    with torch.cuda.device(x1.device):
+    with _on_device(x1.device):
         status = lib.km_dense(
             kid, len(batch_shape), _i64(batch_shape), x1.shape[-1], x2.shape[-1],
             *_tensor_args(x1), *_tensor_args(x2), *_tensor_args(params),
@@ -391,7 +473,7 @@ def dense_bwd(kernel_type: str, x1: Tensor, x2: Tensor, params: Tensor, start: T
     grad = torch.empty((*batch_shape, params.shape[-1]), dtype=torch.float32, device=x1.device)
     need = lib.km_param_grad_workspace_size(kid, len(batch_shape), sizes, m, n, 0)
     workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=x1.device)
-    with torch.cuda.device(x1.device):
+    with _on_device(x1.device):
         status = lib.km_dense_bwd(
             kid, len(batch_shape), sizes, m, n,
             *_tensor_args(x1), *_tensor_args(x2), *_tensor_args(params),
@@ -409,7 +491,10 @@ def make_ranges_2d(x1: Tensor, x2: Tensor | None, cutoff: float, block_size: int
     """Range builders on flattened [batch, n] inputs; result lives on x1's device.
 
     Host tensors go through the sequential host builders, device tensors through the device
-    builders (no host round trip).
+    builders (no host round trip).  The device builders find the scans' results by binary
+    search and therefore require what the pattern itself requires: every row of x1 / x2 sorted
+    ascending.  On unsorted rows the host and device builders return different (equally
+    meaningless) patterns.
     """
     lib = load_library()
     if x1.dtype != torch.float32 or (x2 is not None and x2.dtype != torch.float32):
@@ -422,8 +507,8 @@ def make_ranges_2d(x1: Tensor, x2: Tensor | None, cutoff: float, block_size: int
     end = torch.empty((num_batch, rows), dtype=torch.int32, device=x1.device)
     if x1.is_cuda:
         if x2c is not None and x2c.device != x1c.device:
-            raise RuntimeError("x1 and x2 must be on the same device")
-        with torch.cuda.device(x1.device):
+            x2c = x2c.to(x1c.device)  # the reference accepts mixed devices (it copies both to the host)
+        with _on_device(x1.device):
             if x2c is None:
                 status = lib.km_make_ranges_symmetric_device(
                     _ptr(x1c), num_batch, n1, float(cutoff), block_size, _ptr(start), _ptr(end),

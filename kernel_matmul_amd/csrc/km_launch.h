@@ -39,7 +39,7 @@ struct MatmulProblem {
 
 // Which ahead-of-time instantiation runs and with what decomposition.
 struct MatmulPlan {
-    int variant;     // KM_VARIANT_VALU, KM_VARIANT_MFMA_F32 or KM_VARIANT_MFMA_F16
+    int variant;     // one of the KM_VARIANT_* values above except KM_VARIANT_AUTO
     int k_chunk;     // rhs columns handled per workgroup (MFMA: 16/32/64, VALU: 4/8/16)
     int row_groups;  // MFMA: groups of 16 rows per wavefront (1, 2, 4, 8)
     int col_splits;  // MFMA: wavefronts per workgroup sharing one column range (1, 2, 4, 8)

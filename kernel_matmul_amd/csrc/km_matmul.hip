@@ -1,21 +1,26 @@
 // Forward operator: out = K(x1, x2) @ rhs over per-row-block column ranges, K evaluated on
-// the fly.  Three gfx950 implementations of the same contract (what
-// native/matmul/matmul.cu:13-157 of the reference computes):
+// the fly (what native/matmul/matmul.cu:13-157 of the reference computes).  A wavefront owns
+// whole rows and walks their column range; every x2 / rhs element of the range is loaded once
+// per wavefront, coalesced, straight into MFMA operand layout.  gfx950 implementations of the
+// same contract in this file:
 //
-//   fwd_mfma_f32 : each lane evaluates K entries directly in the A-operand layout of
-//                  v_mfma_f32_16x16x4_f32; the K-tile x rhs-tile contraction is an fp32 MFMA.
-//   fwd_mfma_f16 : K entries and rhs are each split into two fp16 terms (hi + lo, 22
-//                  significant bits) and the contraction is three v_mfma_f32_16x16x32_f16
-//                  (hi*hi + hi*lo + lo*hi) accumulating in fp32.  On gfx950 the fp32 MFMA
-//                  occupies the same issue slots as the VALU that evaluates K, the fp16 MFMA
-//                  does not, so this is the faster variant.
-//   fwd_valu     : one row per lane, contraction with v_fma_f32 on wave-uniform x2 / rhs
-//                  operands fetched through the scalar (read-only) path.
+//   fwd_table_f16 : split-fp16 contraction (below) with per-wavefront column tables in LDS
+//                   (x2, scaled x2, and for spectral kernels cos / sin of the column phases:
+//                   phase-split form).  rbf and spectral kernels, up to 16 rhs columns.  The
+//                   kernel the launch table picks for the headline shape.
+//   fwd_mfma_f16  : K entries and rhs are each split into two fp16 terms (hi + lo, 22
+//                   significant bits); the contraction is three v_mfma_f32_16x16x32_f16
+//                   (hi*hi + hi*lo + lo*hi) accumulating in fp32, K evaluated directly per
+//                   pair.  On gfx950 the fp32 MFMA occupies the same issue slots as the VALU
+//                   that evaluates K, the fp16 MFMA does not.
+//   fwd_mfma_f32  : each lane evaluates K entries in the A-operand layout of
+//                   v_mfma_f32_16x16x4_f32; the contraction is an fp32 MFMA.
+//   fwd_valu      : one row per lane, contraction with v_fma_f32 on wave-uniform x2 / rhs
+//                   operands fetched through the scalar (read-only) path.
 //
-// None of them stages tiles in LDS: a wavefront owns whole rows, so every x2 / rhs element
-// of its column range is loaded once per wavefront, coalesced, straight into the operand
-// layout.  LDS only carries the fixed-order reduction when several wavefronts share a row
-// range.
+// (fwd_block, which prepares the rhs operand once per workgroup of four row blocks, lives in
+// km_matmul_block.hip.)  LDS carries the column tables of fwd_table_f16 and the fixed-order
+// reduction when several wavefronts share a row range.
 #include "km_batch.h"
 #include "km_common.h"
 #include "km_fwd.h"
@@ -23,30 +28,7 @@
 
 namespace km {
 
-
-#ifdef KM_TIMELINE
-// Development aid (never defined in the library build): per-wavefront placement and
-// start/end timestamps for timeline analysis.
-__device__ unsigned long long* g_timeline;
-#define KM_TL_BEGIN() const unsigned long long tl_begin = wall_clock64()
-#define KM_TL_END()                                                                          \
-    do {                                                                                     \
-        if ((threadIdx.x & 63) == 0) {                                                       \
-            const long long tl_id = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6); \
-            g_timeline[tl_id * 4 + 0] = __builtin_amdgcn_s_getreg((31 << 11) | 4);           \
-            g_timeline[tl_id * 4 + 1] = __builtin_amdgcn_s_getreg((3 << 11) | 20);           \
-            g_timeline[tl_id * 4 + 2] = tl_begin;                                            \
-            g_timeline[tl_id * 4 + 3] = wall_clock64();                                      \
-        }                                                                                    \
-    } while (0)
-#else
-#define KM_TL_BEGIN()
-#define KM_TL_END()
-#endif
-
-
-
-// Per-wavefront view of the problem, shared by the three kernels.
+// Per-wavefront view of the problem, shared by the forward kernels.
 struct WaveView {
     long long b;
     int row_block;
@@ -77,7 +59,6 @@ __device__ __forceinline__ WaveView wave_view(const FwdArgs& a, long long item, 
     w.range_end = min(a.end[batch_offset(a.batch, a.end_bs, bidx) + w.row_block * a.end_s], a.n);
     return w;
 }
-
 
 // Work item of this workgroup.  Items are (row chunk, batch item) pairs, contiguous ranges of
 // which belong to one XCD (see xcd_item).  When the launch has a "tail" (only with 128 rows per
@@ -511,7 +492,7 @@ __device__ __forceinline__ void f16_step(const float (&x2v)[8], const float (&ra
 // PF: request the next step's operands before evaluating the current one (costs 8 + 8 G
 // registers; used for G = 1 where they are available).
 template <int KT, int G, int R, bool PF>
-__device__ __forceinline__ void fwd_mfma_f16_body(const FwdArgs& a, float* lds, const WaveView& w,
+__device__ __forceinline__ void fwd_mfma_f16_body(const FwdArgs& a, float* lds, const WaveView& wv,
                                                   int row0) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -519,6 +500,10 @@ __device__ __forceinline__ void fwd_mfma_f16_body(const FwdArgs& a, float* lds, 
     const int li = lane & 15;
     const int kk = lane >> 4;
     const int kbase = blockIdx.y * (16 * G);
+    // The rhs column offset of this workgroup goes into the 64-bit base so that the 32-bit lane
+    // offsets below span at most 24 rows and 16 G columns.
+    WaveView w = wv;
+    w.rhs += (long long)kbase * a.rhs_s1;
 
     const KernelConsts kc = make_consts<KT>(w.params, a.params_s, false);
     const float sigma = w.params[KernelTraits<KT>::SIGMA * a.params_s];
@@ -549,7 +534,7 @@ __device__ __forceinline__ void fwd_mfma_f16_body(const FwdArgs& a, float* lds, 
     for (int g = 0; g < G; g++) {
         const int c = kbase + 16 * g + li;
         colmask[g] = c < a.k;
-        rhs_lane[g] = (unsigned)(8 * kk * a.rhs_s0 + min(c, a.k - 1) * a.rhs_s1);
+        rhs_lane[g] = (unsigned)(8 * kk * a.rhs_s0 + (min(c, a.k - 1) - kbase) * a.rhs_s1);
         // Start far up so that the first non-zero step sets the real scale.
         shift[g] = 100;
         scale[g] = colmask[g] ? __builtin_ldexpf(1.0f, 100) : 0.0f;
@@ -614,7 +599,6 @@ __device__ __forceinline__ void fwd_mfma_f16_body(const FwdArgs& a, float* lds, 
 template <int KT, int G, int R, bool PF>
 __global__ void __launch_bounds__(512) fwd_mfma_f16(const FwdArgs a) {
     extern __shared__ float lds[];
-    KM_TL_BEGIN();
     const ItemRef it = decode_item(a);
     if (!it.valid) {
         return;
@@ -624,13 +608,11 @@ __global__ void __launch_bounds__(512) fwd_mfma_f16(const FwdArgs a) {
         if (it.small) {
             const WaveView w = wave_view(a, it.item, 1, &chunk_in_block);
             fwd_mfma_f16_body<KT, G, 1, false>(a, lds, w, w.row_block * KM_BLOCK_SIZE + 16 * it.piece);
-            KM_TL_END();
             return;
         }
     }
     const WaveView w = wave_view(a, it.item, a.chunks_per_block, &chunk_in_block);
     fwd_mfma_f16_body<KT, G, R, PF>(a, lds, w, w.row_block * KM_BLOCK_SIZE + chunk_in_block * (16 * R));
-    KM_TL_END();
 }
 
 // ---------------------------------------------------------------------------------------
@@ -651,7 +633,6 @@ __global__ void __launch_bounds__(512) fwd_mfma_f16(const FwdArgs a) {
 // ---------------------------------------------------------------------------------------
 #define KM_PHASE_CHUNK 512
 #define KM_PHASE_TABLE_FLOATS (4 * KM_PHASE_CHUNK + KM_PHASE_CHUNK / 32) /* per wavefront */
-
 
 template <int G>
 __device__ __forceinline__ void rhs_load(const FwdArgs& a, const WaveView& w, int c0, int col_end,
@@ -680,7 +661,7 @@ __device__ __forceinline__ void rhs_load(const FwdArgs& a, const WaveView& w, in
 }
 
 template <int KT, int G, int R>
-__device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds, const WaveView& w,
+__device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds, const WaveView& wv,
                                                    int row0) {
     static_assert(KT == KM_KERNEL_SPECTRAL || KT == KM_KERNEL_RBF, "table kernel: rbf or spectral");
     constexpr bool PHASE = KT == KM_KERNEL_SPECTRAL;
@@ -694,6 +675,8 @@ __device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds,
     const int li = lane & 15;
     const int kk = lane >> 4;
     const int kbase = blockIdx.y * (16 * G);
+    WaveView w = wv;  // rhs column offset of this workgroup in the 64-bit base, as above
+    w.rhs += (long long)kbase * a.rhs_s1;
 
     const KernelConsts kc = make_consts<KT>(w.params, a.params_s, false);
     const float sigma = w.params[KernelTraits<KT>::SIGMA * a.params_s];
@@ -722,7 +705,7 @@ __device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds,
 #pragma unroll
     for (int g = 0; g < G; g++) {
         const int c = kbase + 16 * g + li;
-        rhs_lane[g] = (unsigned)(8 * kk * a.rhs_s0 + min(c, a.k - 1) * a.rhs_s1);
+        rhs_lane[g] = (unsigned)(8 * kk * a.rhs_s0 + (min(c, a.k - 1) - kbase) * a.rhs_s1);
         colmask[g] = c < a.k;
         shift[g] = 100;
         scale[g] = c < a.k ? __builtin_ldexpf(1.0f, 100) : 0.0f;
@@ -895,7 +878,6 @@ __device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds,
 template <int KT, int G, int R>
 __global__ void __launch_bounds__(512, 3) fwd_table_f16(const FwdArgs a) {
     extern __shared__ float lds[];
-    KM_TL_BEGIN();
     const ItemRef it = decode_item(a);
     if (!it.valid) {
         return;
@@ -905,13 +887,11 @@ __global__ void __launch_bounds__(512, 3) fwd_table_f16(const FwdArgs a) {
         if (it.small) {
             const WaveView w = wave_view(a, it.item, 1, &chunk_in_block);
             fwd_table_f16_body<KT, G, 1>(a, lds, w, w.row_block * KM_BLOCK_SIZE + 16 * it.piece);
-            KM_TL_END();
             return;
         }
     }
     const WaveView w = wave_view(a, it.item, a.chunks_per_block, &chunk_in_block);
     fwd_table_f16_body<KT, G, R>(a, lds, w, w.row_block * KM_BLOCK_SIZE + chunk_in_block * (16 * R));
-    KM_TL_END();
 }
 
 // ---------------------------------------------------------------------------------------

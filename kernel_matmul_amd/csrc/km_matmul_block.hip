@@ -314,7 +314,9 @@ __global__ void __launch_bounds__(KM_BLK_THREADS, 3) fwd_block(const BlockArgs b
     batch_multi_index(a.batch, b, bidx);
     const float* __restrict__ x1 = a.x1 + batch_offset(a.batch, a.x1_bs, bidx);
     const float* __restrict__ x2 = a.x2 + batch_offset(a.batch, a.x2_bs, bidx);
-    const float* __restrict__ rhs = a.rhs + batch_offset(a.batch, a.rhs_bs, bidx);
+    // The rhs column offset of this workgroup goes into the 64-bit base so that the 32-bit lane
+    // offsets below span at most 24 rows and 16 G columns.
+    const float* __restrict__ rhs = a.rhs + batch_offset(a.batch, a.rhs_bs, bidx) + (long long)kbase * a.rhs_s1;
     const float* __restrict__ params = a.params + batch_offset(a.batch, a.params_bs, bidx);
     const int* __restrict__ start = a.start + batch_offset(a.batch, a.start_bs, bidx);
     const int* __restrict__ end = a.end + batch_offset(a.batch, a.end_bs, bidx);
@@ -395,7 +397,7 @@ __global__ void __launch_bounds__(KM_BLK_THREADS, 3) fwd_block(const BlockArgs b
     for (int g = 0; g < G; g++) {
         shift[g] = 100;
         scale[g] = __builtin_ldexpf(1.0f, 100);
-        rhs_lane[g] = (unsigned)(8 * kk * a.rhs_s0 + min(kbase + 16 * g + li, a.k - 1) * a.rhs_s1);
+        rhs_lane[g] = (unsigned)(8 * kk * a.rhs_s0 + (min(kbase + 16 * g + li, a.k - 1) - kbase) * a.rhs_s1);
     }
     float4v acc[2 * NB][GE];
 #pragma unroll

@@ -119,20 +119,17 @@ except ImportError:
         return device, dtype_
 
 
-def _aligned(start: Tensor, end: Tensor, x2_size: int) -> bool:
-    bad = ((start % _BLOCK_SIZE != 0) & (start != x2_size)) | ((end % _BLOCK_SIZE != 0) & (end != x2_size))
-    return not bool(torch.any(bad))
-
-
 class _MatmulOperator(torch.autograd.Function):
     """K @ rhs with gradients for the hyper-parameters (matmul_bwd) and for rhs (K^T @ grad)."""
 
     @staticmethod
-    def forward(ctx, x1, x2, rhs, params, start, end, native_matmul, native_matmul_bwd, symmetric=False):
+    def forward(ctx, x1, x2, rhs, params, start, end, native_matmul, native_matmul_bwd, symmetric=False,
+                transposed_ranges=None):
         ctx.save_for_backward(x1, x2, rhs, params, start, end)
         ctx.native_matmul = native_matmul
         ctx.native_matmul_bwd = native_matmul_bwd
         ctx.symmetric = symmetric
+        ctx.transposed_ranges = transposed_ranges  # callable returning (start_t, end_t), or None
         return native_matmul(x1, x2, rhs, params, start, end)
 
     @staticmethod
@@ -146,14 +143,18 @@ class _MatmulOperator(torch.autograd.Function):
             if ctx.symmetric:
                 start_t, end_t = start, end
             else:
-                if not _aligned(start, end, x2.shape[-1]):
+                try:
+                    if ctx.transposed_ranges is not None:
+                        start_t, end_t = ctx.transposed_ranges(start.shape[:-1])
+                    else:
+                        start_t, end_t = ranges.transpose_ranges(start, end, x1.shape[-1], x2.shape[-1])
+                except ValueError as error:
                     raise RuntimeError(
                         "the gradient with respect to rhs needs the transposed sparsity pattern; "
                         "build the ranges with align=True"
-                    )
-                start_t, end_t = ranges.transpose_ranges(start, end, x1.shape[-1], x2.shape[-1])
+                    ) from error
             grad_rhs = ctx.native_matmul(x2, x1, grad_output, params, start_t, end_t)
-        return None, None, grad_rhs, grad_params, None, None, None, None, None
+        return None, None, grad_rhs, grad_params, None, None, None, None, None, None
 
 
 class _DenseOperator(torch.autograd.Function):
@@ -234,6 +235,7 @@ class KernelMatmulLinearOperator(LinearOperator):
         self._kernel_type = kernel_type
         self._batch_shape = batch_shape
         self._symmetric = symmetric
+        self._ranges_t = None  # pattern of the transpose, built on first use
 
         self._native_matmul = NativeFunction(
             "matmul", MatmulAutotuneConfiguration(kernel_type), compile_pool=compile_pool
@@ -260,6 +262,20 @@ class KernelMatmulLinearOperator(LinearOperator):
             widen(self._end, 1),
         )
 
+    def _transposed_ranges(self, batch_shape=None) -> tuple[Tensor, Tensor]:
+        """Pattern of K^T, computed once per operator (the check that the pattern is block
+        aligned and the host pass both synchronise with the device); optionally widened to
+        ``batch_shape`` as stride-0 views."""
+        if self._ranges_t is None:
+            self._ranges_t = ranges.transpose_ranges(
+                self._start, self._end, self._x1.size(-2), self._x2.size(-2)
+            )
+        start_t, end_t = self._ranges_t
+        if batch_shape is not None:
+            start_t = start_t.expand(*batch_shape, start_t.shape[-1])
+            end_t = end_t.expand(*batch_shape, end_t.shape[-1])
+        return start_t, end_t
+
     # -- LinearOperator hooks ------------------------------------------------------------
     def _matmul(self, rhs: Tensor) -> Tensor:
         expected = Size((*self._batch_shape, self._x2.size(-2), rhs.size(-1)))
@@ -269,7 +285,7 @@ class KernelMatmulLinearOperator(LinearOperator):
         x1, x2, params, start, end = self._get_args_for_native(batch_shape)
         result = _MatmulOperator.apply(
             x1, x2, rhs_, params, start, end, self._native_matmul, self._native_matmul_bwd,
-            self._symmetric,
+            self._symmetric, self._transposed_ranges,
         )
         return result.reshape(*batch_shape, *result.shape[-2:])
 
@@ -279,9 +295,7 @@ class KernelMatmulLinearOperator(LinearOperator):
     def _transpose_nonbatch(self) -> "KernelMatmulLinearOperator":
         if self._symmetric:
             return self
-        start_t, end_t = ranges.transpose_ranges(
-            self._start, self._end, self._x1.size(-2), self._x2.size(-2)
-        )
+        start_t, end_t = self._transposed_ranges()
         return KernelMatmulLinearOperator(
             self._x2, self._x1, self._params, start_t, end_t, kernel_type=self._kernel_type
         )

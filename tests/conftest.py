@@ -23,6 +23,7 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
     config.addinivalue_line("markers", "square: use x2 = x1 and the symmetric pattern")
     config.addinivalue_line("markers", "align: build block-aligned ranges")
+    config.addinivalue_line("markers", "stable: linspace x, dense pattern, lengthscales x 0.01 (square only)")
 
 
 def pytest_collection_modifyitems(config, items):
@@ -88,15 +89,26 @@ def make_params(kernel_type: str, batch, lengthscale_factor: float = 1.0) -> tor
     return torch.stack(cols, dim=-1).float()
 
 
-def build_example(shape: dict, kernel_type: str, device, square=False, align=False) -> ExampleData:
+def build_example(shape: dict, kernel_type: str, device, square=False, align=False,
+                  stable=False) -> ExampleData:
+    """``stable`` is the regime of the reference's square LinearOperator suite
+    (tests/conftest.py:67-91, 114 there): evenly spaced x, no cutoff (every row block covers all
+    columns) and lengthscales of 0.01 ... 0.02, so that almost every entry of K underflows."""
     from kernel_matmul_amd.ranges import make_ranges
 
+    if stable and not square:
+        pytest.skip("Stable test only implemented for square matrices")
     m = shape["m"]
     n = m if square else shape["n"]
     batch, unsqueeze, k, cutoff = shape["batch"], shape["unsqueeze"], shape["k"], shape["cutoff"]
+    if stable:
+        cutoff = None
     squeeze_batch = batch if unsqueeze is None else (*batch[:unsqueeze], *batch[unsqueeze + 1:])
 
-    x1 = torch.sort(torch.rand(*squeeze_batch, m) * 10, dim=-1)[0]
+    if stable:
+        x1 = torch.linspace(0, 10, m).expand(*squeeze_batch, m)
+    else:
+        x1 = torch.sort(torch.rand(*squeeze_batch, m) * 10, dim=-1)[0]
     x2 = x1 if square else torch.sort(torch.rand(*squeeze_batch, n) * 10, dim=-1)[0]
     if square:
         start, end = make_ranges(cutoff, x1, align=align)
@@ -104,7 +116,7 @@ def build_example(shape: dict, kernel_type: str, device, square=False, align=Fal
         start, end = make_ranges(cutoff, x1, x2, align=align)
     rhs = torch.randn(*squeeze_batch, n, k)
     rhs = rhs / torch.linalg.norm(rhs, dim=-2, keepdim=True)
-    params = make_params(kernel_type, batch)
+    params = make_params(kernel_type, batch, 0.01 if stable else 1.0)
 
     x1, x2, rhs, start, end, params = (t.to(device) for t in (x1, x2, rhs, start, end, params))
     if unsqueeze is not None:
@@ -128,5 +140,7 @@ def example_data(request) -> ExampleData:
     index, kernel_type = request.param
     square = request.node.get_closest_marker("square") is not None
     align = request.node.get_closest_marker("align") is not None
+    stable = request.node.get_closest_marker("stable") is not None
     device = torch.device("cuda:0")
-    return build_example(EXAMPLE_SHAPES[index], kernel_type, device, square=square, align=align)
+    return build_example(EXAMPLE_SHAPES[index], kernel_type, device, square=square, align=align,
+                         stable=stable)

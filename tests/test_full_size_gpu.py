@@ -26,6 +26,7 @@ CONFIGS = {
     "c2": ("spectral", 20_000, 2000.0, 4, 16, 6.0),
     "c3": ("spectral", 50_000, None, 2, 8, 6.0),
     "c3_rbf": ("rbf", 50_000, None, 2, 8, 6.0),
+    "c4": ("spectral", 100_000, 10_000.0, 16, 4, 6.0),
     "headline": ("spectral", 100_000, 10_000.0, 8, 16, 6.0),
     "c5": ("spectral", 1_000_000, 100_000.0, 8, 32, 5.0),
 }
@@ -58,6 +59,59 @@ def _build(name):
     return kernel, n, batch, k, args, host
 
 
+def _banded_matmul_oracle(kernel, h, rhs, batch_items=None):
+    """float64 K @ rhs over the whole pattern, one row block at a time (K never larger than
+    128 x window); rhs is [n, k] shared by the batch or [batch, n, k].  Returns [batch, n, k]."""
+    params = h["params"] if batch_items is None else h["params"][batch_items]
+    nb = params.shape[0]
+    x = h["x"]
+    n = x.shape[0]
+    rhs = np.asarray(rhs, dtype=np.float64)
+    out = np.zeros((nb, n, rhs.shape[-1]))
+    for blk in range(len(h["start"])):
+        r0, r1 = blk * 128, min(blk * 128 + 128, n)
+        s, e = int(h["start"][blk]), min(int(h["end"][blk]), n)
+        if s >= e:
+            continue
+        kb = oracle.kernel_matrix(kernel, np.broadcast_to(x[r0:r1], (nb, r1 - r0)),
+                                  np.broadcast_to(x[s:e], (nb, e - s)), params)
+        seg = rhs[s:e] if rhs.ndim == 2 else (rhs[:, s:e] if batch_items is None else rhs[batch_items][:, s:e])
+        out[:, r0:r1] = kb @ seg
+    return out
+
+
+_FORWARD_ORACLE_CACHE = {}
+
+
+def _forward_oracle(name, kernel, h):
+    """Banded oracle of the configuration's own rhs, computed once per test session (_build is
+    deterministic per name)."""
+    if name not in _FORWARD_ORACLE_CACHE:
+        _FORWARD_ORACLE_CACHE[name] = _banded_matmul_oracle(kernel, h, h["rhs"])
+    return _FORWARD_ORACLE_CACHE[name]
+
+
+def _banded_param_grad_oracle(kernel, h, left, right, batch_items):
+    """float64 gradient of sum((left @ right^T) * masked K) w.r.t. the parameters for the chosen
+    batch items, one row block at a time.  left is [batch, n, c], right [n, c] (shared)."""
+    params = h["params"][batch_items]
+    nb = params.shape[0]
+    x = h["x"]
+    n = x.shape[0]
+    right = np.asarray(right, dtype=np.float64)
+    grad = np.zeros((nb, params.shape[-1]))
+    for blk in range(len(h["start"])):
+        r0, r1 = blk * 128, min(blk * 128 + 128, n)
+        s, e = int(h["start"][blk]), min(int(h["end"][blk]), n)
+        if s >= e:
+            continue
+        g = oracle.kernel_matrix_grad(kernel, np.broadcast_to(x[r0:r1], (nb, r1 - r0)),
+                                      np.broadcast_to(x[s:e], (nb, e - s)), params)
+        coeff = np.asarray(left[batch_items][:, r0:r1], dtype=np.float64) @ right[s:e].T
+        grad += np.einsum("bij,bpij->bp", coeff, g)
+    return grad
+
+
 def _matmul(kernel, a, rhs=None, variant=None):
     rhs = a["rhs"] if rhs is None else rhs
     op_args = (a["x"], a["x"], rhs, a["params"], a["start"], a["end"])
@@ -67,14 +121,16 @@ def _matmul(kernel, a, rhs=None, variant=None):
     return load_native("matmul", defines).call(*op_args)
 
 
-@pytest.mark.parametrize("name,variant", [("c2", None), ("c3_rbf", None), ("headline", None), ("c5", None),
-                                          ("c3_rbf", "block"), ("headline", "block"), ("c5", "block")])
+@pytest.mark.parametrize("name,variant", [("c3_rbf", None), ("c5", None), ("c3_rbf", "block"), ("c5", "block")])
 def test_forward_sampled_blocks_against_oracle(name, variant):
     kernel, n, batch, k, a, h = _build(name)
     out = _matmul(kernel, a, variant=variant)
     assert out.shape == (batch, n, k)
-    blocks = np.unique(np.concatenate([[0, 1, len(h["start"]) - 1],
-                                       np.random.default_rng(1).integers(0, len(h["start"]), 5)]))
+    # first / last blocks, the last 16 row blocks (where the launch cuts items into 16-row
+    # pieces) and a random sample
+    nblk = len(h["start"])
+    blocks = np.unique(np.concatenate([[0, 1], np.arange(max(nblk - 16, 0), nblk),
+                                       np.random.default_rng(1).integers(0, nblk, 48)]))
     for blk in blocks:
         r0, r1 = blk * 128, min(blk * 128 + 128, n)
         s, e = int(h["start"][blk]), int(h["end"][blk])
@@ -86,6 +142,82 @@ def test_forward_sampled_blocks_against_oracle(name, variant):
         got = out[:, r0:r1].cpu().double().numpy()
         err = np.abs(got - expected)
         assert np.all(err <= 1e-5 + 1e-4 * np.abs(expected)), (name, blk, err.max())
+
+
+@pytest.mark.parametrize("name,variant", [("c2", None), ("c3", None), ("headline", None), ("headline", "block"),
+                                          ("headline", "mfma_f32")])
+def test_forward_every_row_block_against_oracle(name, variant):
+    """Every output element of every batch item against the banded float64 oracle."""
+    kernel, n, batch, k, a, h = _build(name)
+    out = _matmul(kernel, a, variant=variant).cpu().double().numpy()
+    expected = _forward_oracle(name, kernel, h)
+    err = np.abs(out - expected)
+    tol = 1e-5 + 1e-4 * np.abs(expected)
+    worst = np.unravel_index(np.argmax(err - tol), err.shape)
+    assert np.all(err <= tol), (name, variant, worst, err[worst], expected[worst])
+
+
+def test_split_fp16_error_against_fp32_mfma_on_headline():
+    """How much accuracy the split-fp16 contraction (the default) trades against the fp32 MFMA
+    contraction, over the full headline output, each against the float64 oracle.  Both must
+    meet rtol 1e-4 / atol 1e-5; the default may be at most 4x worse than the fp32 contraction
+    in worst-case absolute error."""
+    kernel, n, batch, k, a, h = _build("headline")
+    expected = _forward_oracle("headline", kernel, h)
+    errs = {}
+    for variant in (None, "mfma_f32"):
+        out = _matmul(kernel, a, variant=variant).cpu().double().numpy()
+        err = np.abs(out - expected)
+        assert np.all(err <= 1e-5 + 1e-4 * np.abs(expected)), variant
+        errs[variant or "auto"] = (err.max(), (err / (np.abs(expected) + 1e-3)).max())
+    print("max abs / max rel(|expected| + 1e-3) error vs float64:", errs)
+    assert errs["auto"][0] <= 4 * errs["mfma_f32"][0] + 1e-6
+
+
+def test_c3_rhs_and_param_gradients_through_the_operator():
+    """Benchmark configuration 3 asks for the gradients w.r.t. the hyper-parameters and rhs given
+    grad_out [50000, 8]: autograd through KernelMatmulLinearOperator, every element of the rhs
+    gradient and the full parameter gradient against the banded float64 oracle."""
+    from kernel_matmul_amd.linear_operator import KernelMatmulLinearOperator
+
+    for name in ("c3", "c3_rbf"):
+        kernel, n, batch, k, a, h = _build(name)
+        device = a["x"].device
+        params = a["params"].clone().requires_grad_(True)
+        rhs = a["rhs"][0].clone().requires_grad_(True)  # one [n, k] leaf shared by the batch
+        op = KernelMatmulLinearOperator(a["x"][0].unsqueeze(-1), a["x"][0].unsqueeze(-1), params,
+                                        a["start"][0], a["end"][0], kernel_type=kernel, symmetric=True)
+        g = torch.Generator().manual_seed(5)
+        grad_out = torch.randn(batch, n, k, generator=g).to(device)
+        out = op._matmul(rhs)
+        assert out.shape == (batch, n, k)
+        (out * grad_out).sum().backward()
+        # d/d rhs = sum_b K_b^T G_b; the pattern and K are symmetric
+        expected_rhs = _banded_matmul_oracle(kernel, h, grad_out.cpu().numpy()).sum(axis=0)
+        bound = _banded_matmul_oracle(kernel, h, np.abs(grad_out.cpu().numpy())).sum(axis=0)
+        err = np.abs(rhs.grad.cpu().double().numpy() - expected_rhs)
+        assert np.all(err <= 1e-5 + 1e-4 * np.abs(expected_rhs) + 1e-6 * np.abs(bound)), (name, err.max())
+        expected_params = _banded_param_grad_oracle(kernel, h, grad_out.cpu().numpy(), h["rhs"], np.arange(batch))
+        tol = 1e-5 + 1e-4 * np.abs(expected_params).max(axis=-1, keepdims=True)
+        perr = np.abs(params.grad.cpu().double().numpy() - expected_params)
+        assert np.all(perr <= tol), (name, params.grad, expected_params)
+
+
+def test_c4_bilinear_derivative_against_oracle():
+    """Benchmark configuration 4: bilinear derivative, spectral, n = 100000, batch 16, 4 vector
+    columns; the full sums of four batch items against the banded float64 oracle."""
+    kernel, n, batch, k, a, h = _build("c4")
+    g = torch.Generator().manual_seed(6)
+    left = torch.randn(batch, n, k, generator=g).to(a["x"].device)
+    args = (a["x"], a["x"], left, a["rhs"], a["params"], a["start"], a["end"])
+    got = load_native("bilinear_derivative",
+                      BilinearDerivativeConfiguration(kernel).make_config(args)).call(*args)
+    assert got.shape == (batch, 3)
+    items = np.array([0, 5, 10, 15])
+    expected = _banded_param_grad_oracle(kernel, h, left.cpu().numpy(), h["rhs"], items)
+    tol = 1e-5 + 1e-4 * np.abs(expected).max(axis=-1, keepdims=True)
+    err = np.abs(got.cpu().double().numpy()[items] - expected)
+    assert np.all(err <= tol), (got.cpu().numpy()[items], expected)
 
 
 @pytest.mark.parametrize("name", ["headline", "c5"])
@@ -113,7 +245,7 @@ def test_forward_linearity_symmetry_and_variants(name):
         assert torch.allclose(alt, out, rtol=1e-4, atol=float(1e-4 * scale)), variant
 
 
-@pytest.mark.parametrize("name", ["c3", "c3_rbf", "headline"])
+@pytest.mark.parametrize("name", ["c3", "c3_rbf", "c4", "headline"])
 def test_param_grad_identities(name):
     kernel, n, batch, k, a, h = _build(name)
     g = torch.Generator().manual_seed(4)

@@ -116,6 +116,23 @@ def test_matmul_rhs_dynamic_range(example_data, variant):
     assert np.all(err <= tol), float(np.max(err / tol))
 
 
+@pytest.mark.square
+@pytest.mark.stable
+@pytest.mark.parametrize("col_blocks", [1, 2])
+def test_matmul_stable(example_data, col_blocks):
+    """The reference's `stable` regime (its tests/conftest.py:67-91, 114): evenly spaced x, dense
+    pattern, lengthscales of 0.01 ... 0.02."""
+    test_matmul(example_data, col_blocks)
+
+
+@pytest.mark.square
+@pytest.mark.stable
+@pytest.mark.parametrize("variant,rows", [("valu", None), ("mfma_f32", 128), ("mfma_f16", 32), ("mfma_f16", 128),
+                                          ("mfma_f16_direct", 128), ("block", None)])
+def test_matmul_variants_stable(example_data, variant, rows):
+    test_matmul_variants(example_data, variant, rows)
+
+
 def _grad_tolerance(expected):
     # Gradients are sums over up to m*n terms of mixed sign: compare relative to the largest
     # component of each batch item's gradient as well as elementwise.
@@ -151,6 +168,18 @@ def test_bilinear_derivative(example_data):
                                  right.cpu().numpy(), a["params"], a["start"], a["end"])
     err = np.abs(result.cpu().double().numpy() - expected)
     assert np.all(err <= _grad_tolerance(expected)), (result.cpu().numpy(), expected)
+
+
+@pytest.mark.square
+@pytest.mark.stable
+def test_matmul_bwd_stable(example_data):
+    test_matmul_bwd(example_data)
+
+
+@pytest.mark.square
+@pytest.mark.stable
+def test_bilinear_derivative_stable(example_data):
+    test_bilinear_derivative(example_data)
 
 
 @pytest.mark.square
@@ -355,3 +384,154 @@ def test_param_grad_degenerate_ranges(kernel_type):
         expected = oracle.param_grad(kernel_type, f(x1), f(x2), f(out_grad), f(rhs), f(params), f(s), f(e))
         err = np.abs(result.cpu().double().numpy() - expected)
         assert np.all(err <= _grad_tolerance(expected)), (result.cpu().numpy(), expected)
+
+
+def _phase_tolerance(kernel_type, a, rhs64, expected, phase_eps):
+    """rtol * |expected| + (atol + phase_eps) * (envelope @ |rhs|): a phase error of phase_eps
+    radians changes an entry by that fraction of its envelope (the kernel without its
+    oscillating factor), in this library and in the reference alike (both form the phase as an
+    fp32 product frequency * distance)."""
+    if kernel_type == "spectral":
+        env = oracle.dense("rbf", a["x1"], a["x2"], a["params"][..., [0, 2]], a["start"], a["end"])
+    else:  # locally periodic: |dK/dphase| <= (2 / lp) * sigma * exp(-d^2 / (2 l^2))
+        env = oracle.dense("rbf", a["x1"], a["x2"], a["params"][..., [0, 3]], a["start"], a["end"])
+        env = env * np.maximum(1.0, 2.0 / np.abs(a["params"][..., 1, None, None]))
+    return RTOL * np.abs(expected) + (ATOL + phase_eps) * (np.abs(env) @ np.abs(rhs64)) + 1e-30
+
+
+@pytest.mark.parametrize("variant", ["auto", "block", "mfma_f16_direct", "mfma_f32"])
+@pytest.mark.parametrize("frequency", [5.0, 50.0])
+def test_matmul_spectral_high_frequency(frequency, variant):
+    """Spectral kernels with many oscillations per window (up to 125 revolutions across the
+    cutoff) and negative outputscales."""
+    from kernel_matmul_amd.ranges import make_ranges
+
+    g = torch.Generator().manual_seed(21)
+    m, k, batch = 1500, 16, 3
+    x = torch.sort(torch.rand(m, generator=g) * 150.0 + 20.0)[0]
+    start, end = make_ranges(2.5, x)
+    rhs = torch.randn(m, k, generator=g)
+    rhs = rhs / torch.linalg.norm(rhs, dim=-2, keepdim=True)
+    params = torch.stack([1 + torch.rand(batch, generator=g),
+                          frequency * (1 + 0.1 * torch.rand(batch, generator=g)),
+                          torch.tensor([1.5, -0.7, -2.0])], dim=-1)
+    device = torch.device("cuda:0")
+    expand = lambda t: t.to(device).expand(batch, *t.shape)
+    args = (expand(x), expand(x), expand(rhs), params.to(device), expand(start), expand(end))
+    defines = MatmulSingleConfiguration("spectral").make_config(args)
+    defines["MATMUL_VARIANT"] = variant
+    result = load_native("matmul", defines).call(*args).cpu().double().numpy()
+    names = ("x1", "x2", "rhs", "params", "start", "end")
+    a = {name: t.detach().cpu().numpy() for name, t in zip(names, args)}
+    expected = oracle.matmul("spectral", *(a[name] for name in names))
+    # two fp32 roundings of a phase of up to frequency * 1.1 * window revolutions
+    window = float((x[end.long().clamp(max=m) - 1] - x[start.long()]).max())
+    phase_eps = 2 * np.pi * frequency * 1.1 * window * 2.0 ** -23
+    tol = _phase_tolerance("spectral", a, a["rhs"].astype(np.float64), expected, phase_eps)
+    err = np.abs(result - expected)
+    assert np.all(err <= tol), float(np.max(err / tol))
+    assert np.all(np.sign(result[1].sum()) == np.sign(expected[1].sum()))
+
+
+def _far_phase_problem(kernel_type, k):
+    """Long-decay, short-period kernels: the phase frequency * distance reaches thousands of
+    revolutions inside the pattern (the hardware sine / cosine only take +-256)."""
+    g = torch.Generator().manual_seed(31)
+    m, batch = 700, 2
+    x = torch.sort(torch.rand(m, generator=g) * 100.0)[0]
+    if kernel_type == "spectral":
+        params = torch.tensor([[40.0, 30.0, 1.3], [25.0, 47.0, -0.8]])
+        revolutions = 47.0 * 100.0
+    else:
+        params = torch.tensor([[40.0, 1.5, 0.02, 1.3], [25.0, 0.8, 0.011, 0.8]])
+        revolutions = 0.5 / 0.011 * 100.0
+    rows = (m + 127) // 128
+    start = torch.zeros(rows, dtype=torch.int32)
+    end = torch.full((rows,), m, dtype=torch.int32)
+    rhs = torch.randn(m, k, generator=g)
+    rhs = rhs / torch.linalg.norm(rhs, dim=-2, keepdim=True)
+    device = torch.device("cuda:0")
+    expand = lambda t: t.to(device).expand(batch, *t.shape)
+    t = dict(x=expand(x), rhs=expand(rhs), params=params.to(device), start=expand(start), end=expand(end))
+    a = dict(x1=t["x"].cpu().numpy(), x2=t["x"].cpu().numpy(), rhs=t["rhs"].cpu().numpy(),
+             params=params.numpy(), start=t["start"].cpu().numpy(), end=t["end"].cpu().numpy())
+    phase_eps = 2 * np.pi * revolutions * 2.0 ** -23
+    return t, a, phase_eps
+
+
+@pytest.mark.parametrize("kernel_type", ["spectral", "locally_periodic"])
+@pytest.mark.parametrize("variant,k", [("auto", 16), ("auto", 32), ("block", 16), ("mfma_f16_direct", 32),
+                                       ("mfma_f32", 16), ("valu", 8)])
+def test_matmul_phase_beyond_256_revolutions(kernel_type, variant, k):
+    t, a, phase_eps = _far_phase_problem(kernel_type, k)
+    args = (t["x"], t["x"], t["rhs"], t["params"], t["start"], t["end"])
+    defines = MatmulSingleConfiguration(kernel_type).make_config(args)
+    defines["MATMUL_VARIANT"] = variant
+    result = load_native("matmul", defines).call(*args).cpu().double().numpy()
+    expected = oracle.matmul(kernel_type, a["x1"], a["x2"], a["rhs"], a["params"], a["start"], a["end"])
+    tol = _phase_tolerance(kernel_type, a, a["rhs"].astype(np.float64), expected, phase_eps)
+    err = np.abs(result - expected)
+    assert np.all(err <= tol), float(np.max(err / tol))
+
+
+@pytest.mark.parametrize("kernel_type", ["spectral", "locally_periodic"])
+def test_entry_operators_phase_beyond_256_revolutions(kernel_type):
+    """dense, index and the parameter gradient with phases far outside +-256 revolutions."""
+    from kernel_matmul_amd.configurations import DenseConfiguration
+
+    t, a, phase_eps = _far_phase_problem(kernel_type, 5)
+    device = t["x"].device
+    m = a["x1"].shape[-1]
+    one = np.ones((m, 1))
+    kd = oracle.dense(kernel_type, a["x1"], a["x2"], a["params"], a["start"], a["end"])
+    dense_args = (t["x"], t["x"], t["params"], t["start"], t["end"])
+    got = load_native("dense", DenseConfiguration(kernel_type).make_config(dense_args)).call(*dense_args)
+    # per entry: the tolerance of a product with a one-hot rhs
+    if kernel_type == "spectral":
+        env = oracle.dense("rbf", a["x1"], a["x2"], a["params"][..., [0, 2]], a["start"], a["end"])
+    else:
+        env = oracle.dense("rbf", a["x1"], a["x2"], a["params"][..., [0, 3]], a["start"], a["end"])
+        env = env * np.maximum(1.0, 2.0 / np.abs(a["params"][..., 1, None, None]))
+    tol = RTOL * np.abs(kd) + (ATOL + phase_eps) * np.abs(env)
+    err = np.abs(got.cpu().double().numpy() - kd)
+    assert np.all(err <= tol), float(np.max(err / np.maximum(tol, 1e-30)))
+
+    gen = torch.Generator().manual_seed(32)
+    q = 500
+    rows = torch.randint(0, m, (q,), generator=gen, dtype=torch.int32)
+    cols = torch.randint(0, m, (q,), generator=gen, dtype=torch.int32)
+    bi = torch.randint(0, 2, (q,), generator=gen, dtype=torch.int32)
+    iargs = (t["x"], t["x"], t["params"], t["start"], t["end"], (bi.to(device),), rows.to(device), cols.to(device))
+    igot = load_native("index", IndexConfiguration(kernel_type).make_config(iargs)).call(*iargs)
+    sel = (bi.numpy().astype(np.int64), rows.numpy().astype(np.int64), cols.numpy().astype(np.int64))
+    ierr = np.abs(igot.cpu().double().numpy() - kd[sel])
+    assert np.all(ierr <= tol[sel]), float(np.max(ierr / np.maximum(tol[sel], 1e-30)))
+
+    left = torch.randn(2, m, 5, generator=gen)
+    left = (left / torch.linalg.norm(left, dim=-2, keepdim=True)).to(device)
+    gargs = (t["x"], t["x"], left, t["rhs"], t["params"], t["start"], t["end"])
+    ggot = load_native("bilinear_derivative",
+                       BilinearDerivativeConfiguration(kernel_type).make_config(gargs)).call(*gargs)
+    gexp = oracle.param_grad(kernel_type, a["x1"], a["x2"], left.cpu().numpy(), a["rhs"], a["params"],
+                             a["start"], a["end"])
+    # bound of the phase error's effect: sum over pairs of |coefficient| * |d(dK/dtheta)/dphase|;
+    # taken as the sum of |coefficient * dK/dtheta| scaled up by the largest phase sensitivity
+    grads = oracle.kernel_matrix_grad(kernel_type, a["x1"], a["x2"], a["params"])
+    coeff = np.abs(left.cpu().double().numpy() @ np.swapaxes(a["rhs"].astype(np.float64), -1, -2))
+    envg = oracle.kernel_matrix_grad("rbf", a["x1"], a["x2"], a["params"][..., [0, -1]])
+    env_l = np.sum(coeff * np.abs(envg[..., 0, :, :]), axis=(-2, -1))
+    env_s = np.sum(coeff * np.abs(envg[..., 1, :, :]), axis=(-2, -1))
+    dmax = 100.0
+    sig = np.abs(a["params"][..., -1])
+    if kernel_type == "spectral":
+        f = a["params"][..., 1]
+        bound = np.stack([env_l, 2 * np.pi * dmax * sig * env_s * (1 + 0 * f), env_s], axis=-1)
+    else:
+        lp, T = a["params"][..., 1], a["params"][..., 2]
+        amp = np.maximum(1.0, 2.0 / lp)
+        bound = np.stack([env_l * amp, 2 / lp**2 * sig * env_s * amp,
+                          4 * np.pi * dmax / (lp * T**2) * sig * env_s * amp, env_s * amp], axis=-1)
+    gerr = np.abs(ggot.cpu().double().numpy() - gexp)
+    gtol = _grad_tolerance(gexp) + 4 * phase_eps * bound
+    assert np.all(gerr <= gtol), (ggot.cpu().numpy(), gexp, gerr / gtol)
+    del one

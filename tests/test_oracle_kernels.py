@@ -174,3 +174,35 @@ def test_operator_identities(kernel_type):
 
 def test_count_pairs():
     assert oracle.count_pairs(np.array([0, 10]), np.array([100, 50]), 200) == 128 * 100 + 72 * 40
+
+
+@pytest.mark.parametrize("kernel_type", ["rbf", "spectral", "locally_periodic"])
+def test_dense_cpu_baseline_matches_the_float64_oracle(kernel_type):
+    """The fp32 build-K-then-matmul port that bench.py times as the CPU baseline computes the
+    same masked product as the float64 closed forms (fp32 rounding apart), slab by slab."""
+    import torch
+
+    from oracle import dense_cpu
+    from oracle import ranges as oracle_ranges
+
+    g = torch.Generator().manual_seed(17)
+    n, k = 1500, 7
+    x = torch.sort(torch.rand(n, generator=g) * 40.0)[0]
+    params = {"rbf": [1.3, 0.7], "spectral": [1.3, 0.4, 0.7],
+              "locally_periodic": [1.3, 1.1, 1.7, 0.7]}[kernel_type]
+    params = torch.tensor(params)
+    rhs = torch.randn(n, k, generator=g)
+    start, end = oracle_ranges.make_ranges(4.0, x.numpy())
+    expected = oracle.matmul(kernel_type, x.numpy(), x.numpy(), rhs.numpy(), params.numpy(), start, end)
+    st, en = torch.from_numpy(start), torch.from_numpy(end)
+    rows = -(-n // 128)
+    got = torch.cat([dense_cpu.masked_matmul_slab(kernel_type, x, x, rhs, params, st, en, b, min(b + 5, rows))
+                     for b in range(0, rows, 5)])
+    assert got.shape == (n, k)
+    scale = np.abs(oracle.dense(kernel_type, x.numpy(), x.numpy(), params.numpy(), start, end)) @ np.abs(rhs.double().numpy())
+    assert np.all(np.abs(got.double().numpy() - expected) <= 1e-5 * scale + 1e-6)
+    sec, in_band, dense_pairs, slabs, out = dense_cpu.time_masked_matmul(
+        kernel_type, x, x, rhs, params, st, en, budget_seconds=0.0, blocks_per_slab=4)
+    assert slabs == 1 and out.shape == (512, k) and dense_pairs == 512 * n
+    assert in_band == oracle.count_pairs(start[:4], end[:4], 512)
+    assert torch.equal(out, got[:512]) or torch.allclose(out, got[:512], rtol=0, atol=1e-5)
