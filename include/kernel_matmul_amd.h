@@ -142,6 +142,32 @@ int km_param_grad(int kernel_type, int batch_rank, const int64_t* batch_sizes, i
                   float* grad, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------
+ * km_param_grad without any allocation: the same computation with the scratch in a static
+ * device array of KM_STATIC_SCRATCH_BYTES that the library keeps on every GPU it runs on
+ * until the process ends.  No counterpart in the reference (its operators allocate their
+ * scratch with torch::zeros on every call, native/matmul_bwd/matmul_bwd.cu:203-206); it is
+ * for callers that cannot allocate: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  Results are bit-identical to km_param_grad.
+ *   - Problems whose km_param_grad_workspace_size() exceeds KM_STATIC_SCRATCH_BYTES are
+ *     rejected with KM_ERR_WORKSPACE (4 MiB holds 262144 row-block x column-split partial
+ *     rows, e.g. n = 10^6 with batch 32).
+ *   - Every call on one GPU uses that GPU's single array: calls that overlap on one GPU
+ *     (different streams or threads) race; serialise them or use km_param_grad.
+ *   - The first call on a device looks the array's address up (hipGetSymbolAddress); make
+ *     that call outside graph capture.
+ * ---------------------------------------------------------------------------------- */
+#define KM_STATIC_SCRATCH_BYTES (4u << 20)
+
+int km_param_grad_static(int kernel_type, int batch_rank, const int64_t* batch_sizes, int64_t m,
+                         int64_t n, int64_t c, const float* x1, const int64_t* x1_strides,
+                         const float* x2, const int64_t* x2_strides, const float* left,
+                         const int64_t* left_strides, const float* right,
+                         const int64_t* right_strides, const float* params,
+                         const int64_t* params_strides, const int32_t* start,
+                         const int64_t* start_strides, const int32_t* end,
+                         const int64_t* end_strides, float* grad, void* stream);
+
+/* ------------------------------------------------------------------------------------
  * index.  out[q] = K[batch_index_0[q], ..., row_index[q], col_index[q]], 0 outside the mask.
  * Replaces `call` of module km___index___* (native/index/index.cpp:6-24,
  * native/index/index.cu:69-101).  The index tensors share the shape

@@ -92,6 +92,12 @@ def load_library():
         + tensor * 7
         + [_vp, _vp, ctypes.c_size_t, _vp]
     )
+    lib.km_param_grad_static.restype = ctypes.c_int
+    lib.km_param_grad_static.argtypes = (
+        [ctypes.c_int, ctypes.c_int, _i64p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64]
+        + tensor * 7
+        + [_vp, _vp]
+    )
     lib.km_index.restype = ctypes.c_int
     lib.km_index.argtypes = (
         [ctypes.c_int, ctypes.c_int, _i64p, ctypes.c_int64, ctypes.c_int64]
@@ -299,10 +305,14 @@ def matmul(kernel_type: str, x1: Tensor, x2: Tensor, rhs: Tensor, params: Tensor
 
 
 def param_grad(kernel_type: str, x1: Tensor, x2: Tensor, left: Tensor, right: Tensor,
-               params: Tensor, start: Tensor, end: Tensor, out: Tensor | None = None) -> Tensor:
+               params: Tensor, start: Tensor, end: Tensor, out: Tensor | None = None,
+               static_scratch: bool = False) -> Tensor:
     """grad[..., P] of sum((left @ right^T) * K[mask]) w.r.t. params   (C ABI: km_param_grad).
 
-    ``out`` (optional) is a contiguous fp32 tensor [..., P] to write into."""
+    ``out`` (optional) is a contiguous fp32 tensor [..., P] to write into.  With
+    ``static_scratch`` the call goes to km_param_grad_static, which uses the library's per-GPU
+    static scratch instead of a workspace allocated here (together with ``out`` the call then
+    allocates nothing; calls that overlap on one GPU must not both use it)."""
     tensors = (x1, x2, left, right, params, start, end)
     key = _signature("param_grad", kernel_type, tensors)
     prepared = _PREPARED.get(key)
@@ -340,10 +350,14 @@ def param_grad(kernel_type: str, x1: Tensor, x2: Tensor, left: Tensor, right: Te
         call_args.append(t.data_ptr() if filled else None)
         call_args.append(st)
     out_ptr = out.data_ptr() if out.numel() > 0 else None
-    workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=device)
-    with _on_device(device):
-        status = lib.km_param_grad(*head, *call_args, out_ptr, workspace.data_ptr(), need,
-                                   _stream(device))
+    if static_scratch:
+        with _on_device(device):
+            status = lib.km_param_grad_static(*head, *call_args, out_ptr, _stream(device))
+    else:
+        workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=device)
+        with _on_device(device):
+            status = lib.km_param_grad(*head, *call_args, out_ptr, workspace.data_ptr(), need,
+                                       _stream(device))
     if status != 0:
         _raise(lib, status)
     return out

@@ -6,6 +6,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 
 namespace km {
 
@@ -382,18 +383,59 @@ size_t km_param_grad_workspace_size(int kernel_type, int batch_rank, const int64
     return (size_t)nb * (size_t)param_grad_partials_per_batch(m, nb) * KM_MAX_PARAMS * sizeof(float);
 }
 
-int km_param_grad(int kernel_type, int batch_rank, const int64_t* batch_sizes, int64_t m,
-                  int64_t n, int64_t c, const float* x1, const int64_t* x1_strides,
-                  const float* x2, const int64_t* x2_strides, const float* left,
-                  const int64_t* left_strides, const float* right, const int64_t* right_strides,
-                  const float* params, const int64_t* params_strides, const int32_t* start,
-                  const int64_t* start_strides, const int32_t* end, const int64_t* end_strides,
-                  float* grad, void* workspace, size_t workspace_bytes, void* stream) {
-    const char* op = "km_param_grad";
+// Device scratch of the allocation-free entry point: one array per GPU, held until the
+// process ends.  In host code the array's name is only a handle for hipGetSymbolAddress; the
+// address each device keeps it at is looked up once per device and used from then on.
+static __device__ __attribute__((used)) __align__(256) unsigned char scratch[KM_STATIC_SCRATCH_BYTES];
+
+#define KM_MAX_DEVICES 64
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[KM_MAX_DEVICES];  // per device, null until the first call there
+
+// Address of `scratch` on the current device (looked up on the first call per device).
+static int static_scratch(const char* op, void** ptr) {
+    int device = -1;
+    hipError_t err = hipGetDevice(&device);
+    if (err != hipSuccess) return fail_hip(op, err);
+    if (device < 0 || device >= KM_MAX_DEVICES) {
+        return fail(KM_ERR_UNSUPPORTED, "%s: device ordinal %d not supported", op, device);
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[device] == nullptr) {
+        void* p = nullptr;
+        err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (err != hipSuccess || p == nullptr) {
+            return fail_hip(op, err != hipSuccess ? err : hipErrorInvalidSymbol);
+        }
+        g_scratch_ptr[device] = p;
+    }
+    *ptr = g_scratch_ptr[device];
+    return KM_OK;
+}
+
+// Shared body of km_param_grad (caller's workspace) and km_param_grad_static (the library's
+// per-device static scratch).
+static int param_grad_entry(const char* op, bool use_static, int kernel_type, int batch_rank,
+                            const int64_t* batch_sizes, int64_t m, int64_t n, int64_t c,
+                            const float* x1, const int64_t* x1_strides, const float* x2,
+                            const int64_t* x2_strides, const float* left,
+                            const int64_t* left_strides, const float* right,
+                            const int64_t* right_strides, const float* params,
+                            const int64_t* params_strides, const int32_t* start,
+                            const int64_t* start_strides, const int32_t* end,
+                            const int64_t* end_strides, float* grad, void* workspace,
+                            size_t workspace_bytes, void* stream) {
     long long nb = 0;
     if (int rc = check_common(op, kernel_type, batch_rank, batch_sizes, m, n, &nb)) return rc;
     if (c < 0 || c > INT_LIMIT) return fail(KM_ERR_INVALID_ARGUMENT, "%s: c out of range", op);
     if (nb == 0) return KM_OK;
+    const size_t need = km_param_grad_workspace_size(kernel_type, batch_rank, batch_sizes, m, n, c);
+    if (use_static && need > (size_t)KM_STATIC_SCRATCH_BYTES) {
+        return fail(KM_ERR_WORKSPACE,
+                    "%s: this problem needs %zu bytes of scratch, the static buffer holds %zu "
+                    "(use km_param_grad with a caller-provided workspace)",
+                    op, need, (size_t)KM_STATIC_SCRATCH_BYTES);
+    }
     KM_REQUIRE_PTR(op, grad);
     KM_REQUIRE_PTR(op, params);
     KM_REQUIRE_PTR(op, params_strides);
@@ -413,8 +455,9 @@ int km_param_grad(int kernel_type, int batch_rank, const int64_t* batch_sizes, i
         KM_REQUIRE_PTR(op, x2);
         if (c > 0) KM_REQUIRE_PTR(op, right);
     }
-    const size_t need = km_param_grad_workspace_size(kernel_type, batch_rank, batch_sizes, m, n, c);
-    if (need > 0 && (workspace == nullptr || workspace_bytes < need)) {
+    if (use_static) {
+        if (int rc = static_scratch(op, &workspace)) return rc;
+    } else if (need > 0 && (workspace == nullptr || workspace_bytes < need)) {
         return fail(KM_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", op, need,
                     workspace ? workspace_bytes : (size_t)0);
     }
@@ -445,6 +488,33 @@ int km_param_grad(int kernel_type, int batch_rank, const int64_t* batch_sizes, i
     p.workspace = workspace;
     hipError_t err = launch_param_grad(p, (hipStream_t)stream);
     return err == hipSuccess ? KM_OK : fail_hip(op, err);
+}
+
+int km_param_grad(int kernel_type, int batch_rank, const int64_t* batch_sizes, int64_t m,
+                  int64_t n, int64_t c, const float* x1, const int64_t* x1_strides,
+                  const float* x2, const int64_t* x2_strides, const float* left,
+                  const int64_t* left_strides, const float* right, const int64_t* right_strides,
+                  const float* params, const int64_t* params_strides, const int32_t* start,
+                  const int64_t* start_strides, const int32_t* end, const int64_t* end_strides,
+                  float* grad, void* workspace, size_t workspace_bytes, void* stream) {
+    return param_grad_entry("km_param_grad", false, kernel_type, batch_rank, batch_sizes, m, n, c,
+                            x1, x1_strides, x2, x2_strides, left, left_strides, right,
+                            right_strides, params, params_strides, start, start_strides, end,
+                            end_strides, grad, workspace, workspace_bytes, stream);
+}
+
+int km_param_grad_static(int kernel_type, int batch_rank, const int64_t* batch_sizes, int64_t m,
+                         int64_t n, int64_t c, const float* x1, const int64_t* x1_strides,
+                         const float* x2, const int64_t* x2_strides, const float* left,
+                         const int64_t* left_strides, const float* right,
+                         const int64_t* right_strides, const float* params,
+                         const int64_t* params_strides, const int32_t* start,
+                         const int64_t* start_strides, const int32_t* end,
+                         const int64_t* end_strides, float* grad, void* stream) {
+    return param_grad_entry("km_param_grad_static", true, kernel_type, batch_rank, batch_sizes, m, n,
+                            c, x1, x1_strides, x2, x2_strides, left, left_strides, right,
+                            right_strides, params, params_strides, start, start_strides, end,
+                            end_strides, grad, nullptr, 0, stream);
 }
 
 // ---------------------------------------------------------------------------------------

@@ -21,7 +21,7 @@ def declared_functions():
 
 def test_header_declares_the_expected_entry_points():
     names = declared_functions()
-    for required in ("km_matmul", "km_param_grad", "km_param_grad_workspace_size", "km_index",
+    for required in ("km_matmul", "km_param_grad", "km_param_grad_workspace_size", "km_param_grad_static", "km_index",
                      "km_make_ranges", "km_make_ranges_symmetric", "km_transpose_ranges",
                      "km_make_ranges_device", "km_make_ranges_symmetric_device", "km_last_error",
                      "km_version", "km_num_params"):
@@ -73,6 +73,11 @@ def test_device_entry_points_reject_bad_arguments_before_launching():
                          None, None, None, None, None, None, None) == 0
     assert lib.km_param_grad_workspace_size(1, 1, sizes, 1000, 1000, 4) > 0
     assert lib.km_param_grad_workspace_size(1, 1, sizes, 0, 1000, 4) == 0
+    # the allocation-free variant refuses problems beyond its static scratch before anything else
+    many = (ctypes.c_int64 * 1)(64)
+    assert lib.km_param_grad_workspace_size(0, 1, many, 1_000_000, 1_000_000, 2) > 4 << 20
+    status = lib.km_param_grad_static(0, 1, many, 1_000_000, 1_000_000, 2, *([None] * 14), None, None)
+    assert status == -4 and b"static buffer" in lib.km_last_error()
 
 
 def test_missing_library_fails_loudly(monkeypatch):
