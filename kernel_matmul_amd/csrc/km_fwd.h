@@ -59,4 +59,71 @@ __device__ __forceinline__ float phase_rev(float f, float x, float c) {
     return __builtin_fmaf(f, lo, __builtin_fmaf(f, hi, -turns));
 }
 
+// Per-wavefront view of the problem, shared by the forward kernels.
+struct WaveView {
+    long long b;
+    int row_block;
+    const float* x1;
+    const float* x2;
+    const float* rhs;
+    const float* params;
+    int range_start;
+    int range_end;
+};
+
+__device__ __forceinline__ WaveView wave_view(const FwdArgs& a, long long item, int chunks_per_block,
+                                              int* chunk_in_block) {
+    WaveView w;
+    w.b = item % a.num_batches;
+    const int chunk = (int)(item / a.num_batches);
+    w.row_block = chunk / chunks_per_block;
+    *chunk_in_block = chunk % chunks_per_block;
+    int bidx[KM_MAX_BATCH_RANK];
+    batch_multi_index(a.batch, w.b, bidx);
+    w.x1 = a.x1 + batch_offset(a.batch, a.x1_bs, bidx);
+    w.x2 = a.x2 + batch_offset(a.batch, a.x2_bs, bidx);
+    w.rhs = a.rhs + batch_offset(a.batch, a.rhs_bs, bidx);
+    w.params = a.params + batch_offset(a.batch, a.params_bs, bidx);
+    // Clamped to the valid columns: a symmetric pattern over fewer points than one block
+    // reports end = block size > n (native/ranges/ranges.cpp:82-93 of the reference).
+    w.range_start = max(a.start[batch_offset(a.batch, a.start_bs, bidx) + w.row_block * a.start_s], 0);
+    w.range_end = min(a.end[batch_offset(a.batch, a.end_bs, bidx) + w.row_block * a.end_s], a.n);
+    return w;
+}
+
+// Work item of this workgroup.  Items are (row chunk, batch item) pairs, contiguous ranges of
+// which belong to one XCD (see xcd_item).  When the launch has a "tail" (only with 128 rows per
+// wavefront), the last `tail_items` items of every XCD are cut into 8 pieces of 16 rows that are
+// dispatched last: wavefronts are handed out in order, so these short pieces fill the SIMDs
+// that would otherwise idle while others finish a last full-size wavefront.
+struct ItemRef {
+    bool valid;
+    bool small;        // a 16-row piece of a tail item
+    long long item;    // (row chunk, batch) index
+    int piece;         // which 16-row piece (small only)
+};
+
+__device__ __forceinline__ ItemRef decode_item(const FwdArgs& a) {
+    ItemRef it;
+    it.small = false;
+    it.piece = 0;
+    if (a.tail_items == 0) {
+        it.item = xcd_item(blockIdx.x, a.items_per_xcd);
+    } else {
+        const unsigned xcd = blockIdx.x % KM_NUM_XCD;
+        const long long slot = blockIdx.x / KM_NUM_XCD;
+        const long long big = a.items_per_xcd - a.tail_items;
+        if (slot < big) {
+            it.item = (long long)xcd * a.items_per_xcd + slot;
+        } else {
+            const long long t = slot - big;
+            it.small = true;
+            it.item = (long long)xcd * a.items_per_xcd + big + t / 8;
+            it.piece = (int)(t % 8);
+        }
+    }
+    it.valid = it.item < a.total_items;
+    return it;
+}
+
 }  // namespace km

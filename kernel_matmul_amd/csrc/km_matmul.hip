@@ -28,73 +28,6 @@
 
 namespace km {
 
-// Per-wavefront view of the problem, shared by the forward kernels.
-struct WaveView {
-    long long b;
-    int row_block;
-    const float* x1;
-    const float* x2;
-    const float* rhs;
-    const float* params;
-    int range_start;
-    int range_end;
-};
-
-__device__ __forceinline__ WaveView wave_view(const FwdArgs& a, long long item, int chunks_per_block,
-                                              int* chunk_in_block) {
-    WaveView w;
-    w.b = item % a.num_batches;
-    const int chunk = (int)(item / a.num_batches);
-    w.row_block = chunk / chunks_per_block;
-    *chunk_in_block = chunk % chunks_per_block;
-    int bidx[KM_MAX_BATCH_RANK];
-    batch_multi_index(a.batch, w.b, bidx);
-    w.x1 = a.x1 + batch_offset(a.batch, a.x1_bs, bidx);
-    w.x2 = a.x2 + batch_offset(a.batch, a.x2_bs, bidx);
-    w.rhs = a.rhs + batch_offset(a.batch, a.rhs_bs, bidx);
-    w.params = a.params + batch_offset(a.batch, a.params_bs, bidx);
-    // Clamped to the valid columns: a symmetric pattern over fewer points than one block
-    // reports end = block size > n (native/ranges/ranges.cpp:82-93 of the reference).
-    w.range_start = max(a.start[batch_offset(a.batch, a.start_bs, bidx) + w.row_block * a.start_s], 0);
-    w.range_end = min(a.end[batch_offset(a.batch, a.end_bs, bidx) + w.row_block * a.end_s], a.n);
-    return w;
-}
-
-// Work item of this workgroup.  Items are (row chunk, batch item) pairs, contiguous ranges of
-// which belong to one XCD (see xcd_item).  When the launch has a "tail" (only with 128 rows per
-// wavefront), the last `tail_items` items of every XCD are cut into 8 pieces of 16 rows that are
-// dispatched last: wavefronts are handed out in order, so these short pieces fill the SIMDs
-// that would otherwise idle while others finish a last full-size wavefront.
-struct ItemRef {
-    bool valid;
-    bool small;        // a 16-row piece of a tail item
-    long long item;    // (row chunk, batch) index
-    int piece;         // which 16-row piece (small only)
-};
-
-__device__ __forceinline__ ItemRef decode_item(const FwdArgs& a) {
-    ItemRef it;
-    it.small = false;
-    it.piece = 0;
-    if (a.tail_items == 0) {
-        it.item = xcd_item(blockIdx.x, a.items_per_xcd);
-    } else {
-        const unsigned xcd = blockIdx.x % KM_NUM_XCD;
-        const long long slot = blockIdx.x / KM_NUM_XCD;
-        const long long big = a.items_per_xcd - a.tail_items;
-        if (slot < big) {
-            it.item = (long long)xcd * a.items_per_xcd + slot;
-        } else {
-            const long long t = slot - big;
-            it.small = true;
-            it.item = (long long)xcd * a.items_per_xcd + big + t / 8;
-            it.piece = (int)(t % 8);
-        }
-    }
-    it.valid = it.item < a.total_items;
-    return it;
-}
-
 // Fixed-order reduction of the S wavefronts' accumulators through LDS and the masked store.
 // lds[wave][slot][lane], slot = (r * G + g) * 4 + v in the MFMA D layout.
 template <int G, int R>
@@ -320,9 +253,8 @@ __global__ void __launch_bounds__(512) fwd_mfma_f32(const FwdArgs a) {
 // Both scales and sigma are undone on the accumulators before they leave the wavefront.
 // ---------------------------------------------------------------------------------------
 
-// FOLD: x1 holds x1 - r and x2a / x2b hold (x2 - r) * s for a common reference point r, so that
-// u = fma(x1, s, -x2) replaces subtract + multiply (used where both differences are exact).
-template <int KT, bool FOLD = false>
+// KS: log2 of the factor K / sigma is evaluated with (it keeps both halves inside the fp16 range).
+template <int KT, int KS = KM_F16_KSCALE_LOG2>
 __device__ __forceinline__ void kernel_pair_f16(float x1, float x2a, float x2b, const KernelConsts& c,
                                                 float one, half2v* hi, half2v* lo) {
     // Two neighbouring columns at once so that the conversions pack.
@@ -332,8 +264,8 @@ __device__ __forceinline__ void kernel_pair_f16(float x1, float x2a, float x2b, 
 #pragma unroll
     for (int t = 0; t < 2; t++) {
         const float d = x1 - x2s[t];
-        const float u = FOLD ? __builtin_fmaf(x1, c.s, -x2s[t]) : d * c.s;
-        const float arg = __builtin_fmaf(-u, u, (float)KM_F16_KSCALE_LOG2);
+        const float u = d * c.s;
+        const float arg = __builtin_fmaf(-u, u, (float)KS);
         if (KT == KM_KERNEL_RBF) {
             ea[t] = __builtin_amdgcn_exp2f(arg);
             ca[t] = 1.0f;
@@ -357,6 +289,23 @@ __device__ __forceinline__ void kernel_pair_f16(float x1, float x2a, float x2b, 
         // 1.0 that keeps the expression an fma.
         l[t] = (_Float16)__builtin_fmaf(ea[t], KT == KM_KERNEL_SPECTRAL ? ca[t] : one, -(float)h[t]);
     }
+    *hi = h;
+    *lo = l;
+}
+
+// Separable form of the Gaussian factor: 2^(ra * b + rb) for two neighbouring columns, with
+// ra = 2 a, rb = KS - a^2, a = (x1 - r) s the row's and b = (x2 - r) s the columns' scaled
+// distances to a common reference point r; times the columns' 2^(-b^2) (carried by the rhs
+// operand) this is 2^(KS - ((x1 - x2) s)^2).
+__device__ __forceinline__ void separable_pair_f16(float ra, float rb, float ba, float bb, float one,
+                                                   half2v* hi, half2v* lo) {
+    const float ea = __builtin_amdgcn_exp2f(__builtin_fmaf(ra, ba, rb));
+    const float eb = __builtin_amdgcn_exp2f(__builtin_fmaf(ra, bb, rb));
+    const float2v kv = {ea, eb};
+    const half2v h = __builtin_convertvector(kv, half2v);
+    half2v l;
+    l[0] = (_Float16)__builtin_fmaf(ea, one, -(float)h[0]);
+    l[1] = (_Float16)__builtin_fmaf(eb, one, -(float)h[1]);
     *hi = h;
     *lo = l;
 }
@@ -413,8 +362,10 @@ __device__ __forceinline__ void f16_load(const FwdArgs& a, const WaveView& w, in
 // row group evaluate 8 kernel entries, split them and issue the three MFMAs.
 // PARTS = 2 (phase-split form): every rhs value enters twice, multiplied by cb[] and by sb[]
 // (|cb|, |sb| <= 1), into the accumulator groups g and G + g; both share the column's scale,
-// which is taken from |rhs| alone.
-template <int KT, int G, int R, bool FOLD = false, int PARTS = 1>
+// which is taken from |rhs| alone.  PARTS = 1 with MULT: every rhs value is multiplied by cb[].
+// SEP: x2v holds b = (x2 - ref) s and the entries are evaluated in the separable form (their
+// column factors 2^(-b^2) come in through cb / sb).
+template <int KT, int G, int R, int KS = KM_F16_KSCALE_LOG2, bool SEP = false, int PARTS = 1, bool MULT = false>
 __device__ __forceinline__ void f16_step(const float (&x2v)[8], const float (&raw)[G][8],
                                          const float (&x1v)[R], const KernelConsts& kc,
                                          const bool (&colmask)[G], int (&shift)[G],
@@ -438,7 +389,7 @@ __device__ __forceinline__ void f16_step(const float (&x2v)[8], const float (&ra
             if (grow) {
                 // m < 2^e, so m * 2^(14 - e) < 2^14.
                 const int e = __builtin_amdgcn_frexp_expf(m);
-                const int new_shift = min(max(KM_F16_KSCALE_LOG2 - e, -100), 100);
+                const int new_shift = min(max(14 - e, -100), 100);
                 const float factor = __builtin_ldexpf(1.0f, new_shift - shift[g]);
 #pragma unroll
                 for (int r = 0; r < R; r++) {
@@ -466,6 +417,12 @@ __device__ __forceinline__ void f16_step(const float (&x2v)[8], const float (&ra
             split_f16x8(vc, kc.one, &bhi[g], &blo[g]);
             split_f16x8(vs, kc.one, &bhi[G + g], &blo[G + g]);
         } else {
+            if (MULT) {
+#pragma unroll
+                for (int t = 0; t < 8; t++) {
+                    rv[t] *= cb[t];
+                }
+            }
             split_f16x8(rv, kc.one, &bhi[g], &blo[g]);
         }
     }
@@ -473,10 +430,20 @@ __device__ __forceinline__ void f16_step(const float (&x2v)[8], const float (&ra
 #pragma unroll
     for (int r = 0; r < R; r++) {
         half2v h2[4], l2[4];
-        const float x1 = FOLD ? x1v[r] - ref : x1v[r];  // FOLD: relative to the step's reference point
+        if (SEP) {
+            // Row constants for this lane's 8 columns (ref: their reference point).
+            const float av = (x1v[r] - ref) * kc.s;
+            const float ra = av + av;
+            const float rb = __builtin_fmaf(-av, av, (float)KS);
 #pragma unroll
-        for (int t = 0; t < 4; t++) {
-            kernel_pair_f16<KT, FOLD>(x1, x2v[2 * t], x2v[2 * t + 1], kc, kc.one, &h2[t], &l2[t]);
+            for (int t = 0; t < 4; t++) {
+                separable_pair_f16(ra, rb, x2v[2 * t], x2v[2 * t + 1], kc.one, &h2[t], &l2[t]);
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                kernel_pair_f16<KT, KS>(x1v[r], x2v[2 * t], x2v[2 * t + 1], kc, kc.one, &h2[t], &l2[t]);
+            }
         }
         const half8v ahi = join_half2x4(h2);
         const half8v alo = join_half2x4(l2);
@@ -485,6 +452,11 @@ __device__ __forceinline__ void f16_step(const float (&x2v)[8], const float (&ra
             acc[r][g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahi, bhi[g], acc[r][g], 0, 0, 0);
             acc[r][g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahi, blo[g], acc[r][g], 0, 0, 0);
             acc[r][g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(alo, bhi[g], acc[r][g], 0, 0, 0);
+        }
+        if (SEP) {
+            // One row group at a time: the row constants of later groups are not formed ahead
+            // of their use (registers); the MFMAs still overlap the next group's evaluation.
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 }
@@ -616,23 +588,57 @@ __global__ void __launch_bounds__(512) fwd_mfma_f16(const FwdArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------
-// Spectral kernel, phase-split form of the split-fp16 variant.
+// Table kernel (rbf and spectral, up to 16 rhs columns): split-fp16 contraction with
+// per-wavefront column tables in LDS.
 //
-// With a reference point c per wavefront (its first row) and A_i = 2 pi f (x1_i - c),
-// B_j = 2 pi f (x2_j - c):
+// Phase-split form (spectral).  With a reference point c per wavefront (its first row) and
+// A_i = 2 pi f (x1_i - c), B_j = 2 pi f (x2_j - c):
 //     cos(2 pi f (x1_i - x2_j)) = cos A_i cos B_j + sin A_i sin B_j
 //     out[i,:] = cos A_i * sum_j E_ij (cos B_j rhs[j,:]) + sin A_i * sum_j E_ij (sin B_j rhs[j,:])
-// with E_ij = exp(-d^2 / (2 l^2)) the Gaussian factor alone.  The cosine leaves the per-pair
-// work: a pair costs sub, mul, fma, exp2 and the hi/lo split (5 full-rate + 1 transcendental
-// instructions instead of 7 + 2), in exchange for twice the fp16 MFMAs, which run beside the
-// VALU.  cos B_j / sin B_j are needed once per column: each chunk of 512 columns is tabulated
-// cooperatively by the wavefront (8 columns per lane) into LDS together with x2, and the
-// steps read their 8 columns back as broadcast vector reads.  Phases are formed from an exact
-// two-term difference to the reference point (once per row / column), so they are accurate to
-// 3e-8 revolutions for any window width.
+// with E_ij = exp(-d^2 / (2 l^2)) the Gaussian factor alone: the cosine leaves the per-pair
+// work in exchange for twice the fp16 MFMAs.  cos B_j / sin B_j are needed once per column:
+// each chunk of 512 columns is tabulated cooperatively by the wavefront (8 columns per lane)
+// into LDS, and the steps read their 8 columns back as broadcast vector reads.  Phases are
+// formed from an exact two-term difference to the reference point (once per row / column), so
+// they are accurate to 3e-8 revolutions for any window width.
+//
+// Separable exponent.  A lane evaluates, per step, its row against 8 consecutive columns.
+// With r the x2 value in the middle of these 8 columns, a = (x1_i - r) s and b_j = (x2_j - r) s:
+//     2^(S - (a - b_j)^2) = 2^((S - a^2) + 2 a b_j) * 2^(-b_j^2)
+// The last factor depends on the column alone and is tabulated with cos B_j / sin B_j (it
+// multiplies the rhs operand); what is left per pair is ONE fma and one exp2, with the two row
+// constants 2 a and S - a^2 formed once per row and 8 columns.  A chunk takes this form only
+// when it loses nothing: every x2_j - r must be exact in fp32 (error-free transformation),
+// every x1_i - r too (all coordinates involved have one sign and a spread below their smallest
+// magnitude), and |b_j| <= 2, which bounds the evaluated factor by 2^(S + 4) -- inside the
+// fp16 range for S = 11 -- and the column factor from below by 2^-4.  Otherwise (coordinates
+// next to the origin, unsorted or widely spaced columns) the chunk evaluates
+// 2^(S - ((x1_i - x2_j) s)^2) directly.
 // ---------------------------------------------------------------------------------------
 #define KM_PHASE_CHUNK 512
-#define KM_PHASE_TABLE_FLOATS (4 * KM_PHASE_CHUNK + KM_PHASE_CHUNK / 32) /* per wavefront */
+#define KM_PHASE_TABLE_FLOATS (4 * KM_PHASE_CHUNK + KM_PHASE_CHUNK / 8) /* per wavefront */
+#define KM_TABLE_KSCALE_LOG2 11
+#define KM_TABLE_SPAN 2.0f
+
+// Minimum and maximum over the wavefront, returned wave-uniform.  Row-wise DPP steps, then the
+// last lane of each row of 16 is carried into the following rows; lane 63 holds the result.
+__device__ __forceinline__ void wave_min_max(float* lo, float* hi) {
+    float a = *lo, b = *hi;
+#define KM_DPP_STEP(ctrl)                                                                              \
+    a = fminf(a, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, a),     \
+                                                                       __builtin_bit_cast(int, a), ctrl, 0xf, 0xf, false))); \
+    b = fmaxf(b, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, b),     \
+                                                                       __builtin_bit_cast(int, b), ctrl, 0xf, 0xf, false)))
+    KM_DPP_STEP(0xb1);   // quad_perm [1, 0, 3, 2]
+    KM_DPP_STEP(0x4e);   // quad_perm [2, 3, 0, 1]
+    KM_DPP_STEP(0x114);  // row_shr 4
+    KM_DPP_STEP(0x118);  // row_shr 8
+    KM_DPP_STEP(0x142);  // row_bcast 15
+    KM_DPP_STEP(0x143);  // row_bcast 31
+#undef KM_DPP_STEP
+    *lo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, a), 63));
+    *hi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, b), 63));
+}
 
 template <int G>
 __device__ __forceinline__ void rhs_load(const FwdArgs& a, const WaveView& w, int c0, int col_end,
@@ -668,6 +674,8 @@ __device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds,
     // Accumulator groups; phase-split: [cos part of g = 0..G), sin part of g = 0..G)].
     constexpr int GE = PHASE ? 2 * G : G;
     constexpr int CH = KM_PHASE_CHUNK;
+    constexpr int PER_LANE = CH / 64;
+    constexpr int KS = KM_TABLE_KSCALE_LOG2;
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -720,20 +728,16 @@ __device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds,
         }
     }
 
-    // Per-wavefront table of the current chunk: x2, cos B, sin B, and for the folded form
-    // (x2 - r) * s with r the x2 value in the middle of each step of 32 columns.
+    // Per-wavefront table of the current chunk: x2, b = (x2 - r) s with r the x2 value in the
+    // middle of each group of 8 columns, the two column factors of the rhs operand (cos B and
+    // sin B, times 2^(-b^2) in the separable form; rbf: the first alone), and the r's.
     float* tab_x2 = lds + (size_t)wave * KM_PHASE_TABLE_FLOATS;
-    float* tab_cos = tab_x2 + CH;
+    float* tab_b = tab_x2 + CH;
+    float* tab_cos = tab_b + CH;
     float* tab_sin = tab_cos + CH;
-    float* tab_xs = tab_sin + CH;
-    float* tab_ref = tab_xs + CH;
+    float* tab_ref = tab_sin + CH;
     float* reduce_buffer = lds + (size_t)S * KM_PHASE_TABLE_FLOATS;
 
-    // Folded form u = fma(x1 - r, s, -[(x2 - r) s]): one instruction less per pair.  A chunk
-    // uses it only if it loses nothing: every x2 - r must be exact (error-free transformation),
-    // every x1 - r too (all coordinates involved are multiples of the ulp of the smallest
-    // magnitude, so a spread below that magnitude is sufficient), and |(x2 - r) s| <= 16 keeps
-    // the one rounding of the tabulated product below 1e-6.
     float row_lo = __builtin_inff(), row_hi = -__builtin_inff();
     bool row_nan = false;
 #pragma unroll
@@ -742,95 +746,146 @@ __device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds,
         row_hi = fmaxf(row_hi, x1v[r]);
         row_nan = row_nan || x1v[r] != x1v[r];
     }
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        row_lo = fminf(row_lo, __shfl_xor(row_lo, off, 64));
-        row_hi = fmaxf(row_hi, __shfl_xor(row_hi, off, 64));
-    }
+    wave_min_max(&row_lo, &row_hi);
     const bool rows_finite = !__any(row_nan);
-    row_lo = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, row_lo)));
-    row_hi = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, row_hi)));
 
-    for (int chunk0 = col_begin; chunk0 < col_end; chunk0 += CH) {
+    // Tabulates the chunk [chunk0, chunk0 + 512) of this wavefront's columns; returns whether it
+    // may take the separable form (then, if `allow`, the column factors already carry 2^(-b^2)).
+    auto build = [&](int chunk0, bool allow) -> bool {
         const int chunk_end = min(chunk0 + CH, col_end);
         const int padded = (chunk_end - chunk0 + 31) & ~31;
-        bool cols_ok = true;
-        float lo = row_lo, hi = row_hi;
         // Strides are below 2^24 elements, so 32 x 32 -> 64 bit products are enough.
         const float* x2c = w.x2 + (long long)chunk0 * a.x2_s;
         const unsigned x2_stride = (unsigned)a.x2_s;
         const int last = chunk_end - 1 - chunk0;
-        for (int q = lane; q < padded; q += 64) {
-            const float xv = x2c[(unsigned long long)(unsigned)min(q, last) * x2_stride];
-            const float ref = x2c[(unsigned long long)(unsigned)min((q & ~31) + 16, last) * x2_stride];
-            const float xd = xv - ref;
-            const float bb = xd - xv;
-            const float err = (xv - (xd - bb)) - (ref + bb);  // exact rounding error of xd
-            const float xs = xd * kc.s;
-            tab_x2[q] = xv;
-            if (PHASE) {
-                const float th = phase_rev(kc.f, xv, c_ref);
-                tab_cos[q] = __builtin_amdgcn_cosf(th);
-                tab_sin[q] = __builtin_amdgcn_sinf(th);
-            }
-            tab_xs[q] = xs;
-            if ((q & 31) == 0) {
-                tab_ref[q >> 5] = ref;
-            }
-            cols_ok = cols_ok && err == 0.0f && fabsf(xs) <= 16.0f;
-            lo = fminf(lo, ref);
-            hi = fmaxf(hi, ref);
-        }
+        // All loads of the chunk are requested before any is used: this lane's 8 columns
+        // (lane, lane + 64, ...) and the reference point of column group `lane`; they go
+        // straight to LDS, the arithmetic on them runs from there (few registers).
+        {
+            float xq[PER_LANE];
 #pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            lo = fminf(lo, __shfl_xor(lo, off, 64));
-            hi = fmaxf(hi, __shfl_xor(hi, off, 64));
+            for (int i = 0; i < PER_LANE; i++) {
+                xq[i] = x2c[(unsigned long long)(unsigned)min(lane + 64 * i, last) * x2_stride];
+            }
+            const float ref_own = x2c[(unsigned long long)(unsigned)min(8 * lane + 4, last) * x2_stride];
+#pragma unroll
+            for (int i = 0; i < PER_LANE; i++) {
+                tab_x2[lane + 64 * i] = xq[i];
+            }
+            tab_ref[lane] = ref_own;
         }
-        const bool rows_ok = rows_finite && (lo > 0.0f || hi < 0.0f) && (hi - lo) <= fminf(fabsf(lo), fabsf(hi));
-        const bool fold = __all(cols_ok) && rows_ok;
-        // The table is written and read by this wavefront only.
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-        auto steps = [&](auto fold_c) {
-            constexpr bool FOLD = decltype(fold_c)::value;
-            float raw[G][8];
-            rhs_load<G>(a, w, chunk0, chunk_end, kk, rhs_lane, raw);
-            for (int c0 = chunk0; c0 < chunk_end; c0 += 32) {
-                const int off = c0 - chunk0 + 8 * kk;
-                float x2v[8], cb[8], sb[8];
-#pragma unroll
-                for (int t = 0; t < 8; t += 4) {
-                    const float4v vx = *(const float4v*)((FOLD ? tab_xs : tab_x2) + off + t);
-#pragma unroll
-                    for (int u = 0; u < 4; u++) {
-                        x2v[t + u] = vx[u];
-                    }
-                    if (PHASE) {
-                        const float4v vc = *(const float4v*)(tab_cos + off + t);
-                        const float4v vs = *(const float4v*)(tab_sin + off + t);
-#pragma unroll
-                        for (int u = 0; u < 4; u++) {
-                            cb[t + u] = vc[u];
-                            sb[t + u] = vs[u];
-                        }
-                    }
-                }
-                const float ref = FOLD ? tab_ref[(c0 - chunk0) >> 5] : 0.0f;
-                f16_step<KM_KERNEL_RBF, G, R, FOLD, GE / G>(x2v, raw, x1v, kc, colmask, shift, scale, acc, ref, cb, sb);
-                if (c0 + 32 < chunk_end) {
-                    rhs_load<G>(a, w, c0 + 32, chunk_end, kk, rhs_lane, raw);
+        bool cols_ok = true;
+        float lo = row_lo, hi = row_hi;
+#pragma unroll 1
+        for (int q = lane; q < padded; q += 64) {
+            const float xv = tab_x2[q];
+            const float ref = tab_ref[q >> 3];
+            const float xd = xv - ref;
+            const float bb = xd - xv;
+            const float err = (xv - (xd - bb)) - (ref + bb);  // exact rounding error of xd
+            const float b = xd * kc.s;
+            tab_b[q] = b;
+            if (PHASE) {
+                const float th = phase_rev(kc.f, xv, c_ref);
+                tab_cos[q] = __builtin_amdgcn_cosf(th);
+                tab_sin[q] = __builtin_amdgcn_sinf(th);
+            } else {
+                tab_cos[q] = 1.0f;
+            }
+            cols_ok = cols_ok && err == 0.0f && fabsf(b) <= KM_TABLE_SPAN;
+            lo = fminf(lo, ref);
+            hi = fmaxf(hi, ref);
+        }
+        wave_min_max(&lo, &hi);
+        // x1 - r is exact for every row and reference point when all coordinates involved have
+        // one sign and their spread does not exceed the smallest magnitude.
+        const bool rows_ok = rows_finite && (lo > 0.0f || hi < 0.0f) && (hi - lo) <= fminf(fabsf(lo), fabsf(hi));
+        const bool separable = allow && __all(cols_ok) && rows_ok;
+        if (separable) {
+            // The column factor 2^(-b^2) of the separable form joins the phase factors.
+#pragma unroll 1
+            for (int q = lane; q < padded; q += 64) {
+                const float b = tab_b[q];
+                const float wgt = __builtin_amdgcn_exp2f(-b * b);
+                tab_cos[q] *= wgt;
+                if (PHASE) {
+                    tab_sin[q] *= wgt;
                 }
             }
-        };
-        if (fold) {
-            steps(std::integral_constant<bool, true>{});
-        } else {
-            steps(std::integral_constant<bool, false>{});
         }
+        // The table is written and read by this wavefront only.
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        return separable;
+    };
+
+    // The steps of a tabulated chunk.
+    auto steps = [&](int chunk0, auto sep_c) {
+        constexpr bool SEP = decltype(sep_c)::value;
+        const int chunk_end = min(chunk0 + CH, col_end);
+        float raw[G][8];
+        rhs_load<G>(a, w, chunk0, chunk_end, kk, rhs_lane, raw);
+        for (int c0 = chunk0; c0 < chunk_end; c0 += 32) {
+            const int off = c0 - chunk0 + 8 * kk;
+            float x2v[8], cb[8], sb[8];
+#pragma unroll
+            for (int t = 0; t < 8; t += 4) {
+                const float4v vx = *(const float4v*)((SEP ? tab_b : tab_x2) + off + t);
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    x2v[t + u] = vx[u];
+                }
+                if (PHASE || SEP) {
+                    const float4v vc = *(const float4v*)(tab_cos + off + t);
+#pragma unroll
+                    for (int u = 0; u < 4; u++) {
+                        cb[t + u] = vc[u];
+                    }
+                }
+                if (PHASE) {
+                    const float4v vs = *(const float4v*)(tab_sin + off + t);
+#pragma unroll
+                    for (int u = 0; u < 4; u++) {
+                        sb[t + u] = vs[u];
+                    }
+                }
+            }
+            const float ref = SEP ? tab_ref[off >> 3] : 0.0f;
+            f16_step<KM_KERNEL_RBF, G, R, KS, SEP, GE / G, SEP && !PHASE>(x2v, raw, x1v, kc, colmask, shift,
+                                                                        scale, acc, ref, cb, sb);
+            if (c0 + 32 < chunk_end) {
+                rhs_load<G>(a, w, c0 + 32, chunk_end, kk, rhs_lane, raw);
+            }
+        }
+        // All reads of the table are done before the next chunk overwrites it.
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    };
+
+    // Separable chunks first; from the first chunk that cannot take that form on, the rest of
+    // the range is evaluated directly (two loops in sequence rather than a choice inside one
+    // loop: the register allocation of each stays on its own).
+    int chunk0 = col_begin;
+    bool tabulated = false;
+    for (; chunk0 < col_end; chunk0 += CH) {
+        tabulated = true;
+        if (!build(chunk0, true)) {
+            break;
+        }
+        steps(chunk0, std::integral_constant<bool, true>{});
+        tabulated = false;
+    }
+    for (; chunk0 < col_end; chunk0 += CH) {
+        if (!tabulated) {
+            build(chunk0, false);
+        }
+        tabulated = false;
+        steps(chunk0, std::integral_constant<bool, false>{});
     }
 
     // Power-of-two scales undone and sigma applied; phase-split:
@@ -853,7 +908,7 @@ __device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds,
         }
 #pragma unroll
         for (int g = 0; g < G; g++) {
-            const float up = __builtin_ldexpf(sigma, -shift[g] - KM_F16_KSCALE_LOG2);
+            const float up = __builtin_ldexpf(sigma, -shift[g] - KS);
 #pragma unroll
             for (int v = 0; v < 4; v++) {
                 if (PHASE) {
