@@ -1,19 +1,21 @@
 #!/usr/bin/env python3
 """Headline benchmark: sparse spectral K(x, x) @ rhs, n = 100 000, k = 16, batch 8, one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload headline|c1|c2|c5]
-                    [--variant auto|mfma|valu] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload headline|c1|...|ref_example]
+                    [--variant auto|...] [--no-cpu-baseline] [--no-configs]
 
-A step is one call of the matmul operator over the whole batch with inputs resident in HBM.
+A step is one call of the operator over the whole batch with inputs resident in HBM.
 Prints one JSON line: kernel-pair evaluations per second (``value``), the roofline of the
-forward kernel against the MI355X fp32 peak (157.3 TFLOP/s, vector = matrix fp32), and the
-CPU baseline (dense build-K-then-matmul in fp32 torch on the host cores, bounded sample).
+forward kernel against the MI355X fp32 peak (157.3 TFLOP/s, vector = matrix fp32), the same
+figures for every other benchmark configuration (``configs``), the error of the default
+(split-fp16) and of the fp32-MFMA contraction against a float64 evaluation of the whole output
+(``roofline.error_vs_fp64``), and the CPU baseline (dense build-K-then-matmul in fp32 torch on
+the host cores, bounded sample).
 """
 from __future__ import annotations
 
 import argparse
 import json
-import math
 import os
 import sys
 import time
@@ -34,13 +36,20 @@ WORKLOADS = {
                label="spectral K@rhs n=20000 k=16 batch=4 cutoff=6*l_max"),
     "c3": dict(kernel="spectral", n=50_000, extent=None, batch=2, k=8, cutoff_l=6.0, seed=1003, op="param_grad",
                label="spectral matmul_bwd n=50000 k=8 batch=2 x=cumsum(Exp(1)) cutoff=6*l_max"),
+    "c3_rhs_grad": dict(kernel="spectral", n=50_000, extent=None, batch=2, k=8, cutoff_l=6.0, seed=1003,
+                        label="spectral rhs gradient (K^T @ grad_out) n=50000 k=8 batch=2 x=cumsum(Exp(1))"),
     "c4": dict(kernel="spectral", n=100_000, extent=10_000.0, batch=16, k=4, cutoff_l=6.0, seed=1004, op="param_grad",
                label="spectral bilinear_derivative n=100000 d=4 batch=16 cutoff=6*l_max"),
     "c5": dict(kernel="spectral", n=1_000_000, extent=100_000.0, batch=8, k=32, cutoff_l=5.0, seed=1005,
                label="spectral K@rhs n=1000000 k=32 batch=8 cutoff=5*l_max"),
+    # the reference's own benchmark recipe (examples/matmul.py:61-82 there)
+    "ref_example": dict(kernel="rbf", n=65_536, extent=65_536 / 24.0, batch=1, k=64, cutoff_abs=10.0, seed=0,
+                        label="rbf K@rhs n=65536 k=64 batch=1 x~U[0,n/24) cutoff=10 params=1+0.01*N(0,1)"),
 }
 
-# (FETCH_SIZE 3543.6 KiB x 2.00 + WRITE_SIZE 50000.0 KiB x 1.00) x 1024
+# HBM bytes per launch of the headline kernel, from the FETCH_SIZE / WRITE_SIZE counter runs
+# summarised in the file named here (an offline rocprofv3 --pmc run, not measured by this script).
+TRAFFIC_SOURCE = "profiles/fwd_table_f16_headline_counters.md"
 MEASURED_TRAFFIC_BYTES = {"headline": 58763674}
 
 FLOPS_PER_PAIR = {"rbf": lambda k: 5 + 2 * k, "spectral": lambda k: 8 + 2 * k,
@@ -64,13 +73,136 @@ def make_workload(name: str, batch_override=None):
         x = torch.sort(torch.rand(n, generator=g) * w["extent"])[0]
     bshape = (batch,) if batch else ()
     u = lambda lo, hi: lo + (hi - lo) * torch.rand(bshape, generator=g)
-    if w["kernel"] == "spectral":
+    if name == "ref_example":
+        params = 1.0 + 0.01 * torch.randn(*bshape, 2, generator=g)
+    elif w["kernel"] == "spectral":
         params = torch.stack([u(0.5, 2.0), u(0.05, 0.5), u(0.5, 2.0)], dim=-1)
     else:
         params = torch.stack([torch.ones(bshape), torch.ones(bshape)], dim=-1)
     rhs = torch.randn(n, w["k"], generator=g)
+    if name == "ref_example":
+        rhs = rhs / rhs.norm(dim=0, keepdim=True)
     cutoff = w["cutoff_abs"] if "cutoff_abs" in w else w["cutoff_l"] * float(params[..., 0].max())
     return w, x, params.float(), rhs, cutoff
+
+
+class Prepared:
+    """One workload resident on the GPU, ready to be called."""
+
+    def __init__(self, name, device, batch_override=None, variant="auto", rows_per_wave=0, col_splits=0,
+                 tail_balance=True):
+        import torch
+
+        from kernel_matmul_amd.compile import load_native
+        from kernel_matmul_amd.configurations import BilinearDerivativeConfiguration, MatmulSingleConfiguration
+        from kernel_matmul_amd.ranges import make_ranges
+
+        self.name = name
+        self.w, self.x_cpu, self.params_cpu, self.rhs_cpu, self.cutoff = make_workload(name, batch_override)
+        w = self.w
+        n, k, batch = w["n"], w["k"], w["batch"]
+        bshape = (batch,) if batch else ()
+        self.start_cpu, self.end_cpu = make_ranges(self.cutoff, self.x_cpu)  # symmetric pattern, block 128
+        row_blocks = self.start_cpu.shape[-1]
+        rows_in_block = torch.clamp(n - 128 * torch.arange(row_blocks), max=128)
+        self.pairs = int((rows_in_block * (self.end_cpu - self.start_cpu)).sum()) * max(batch, 1)
+        self.is_grad = w.get("op") == "param_grad"
+        self.flops_per_pair = (GRAD_FLOPS_PER_PAIR if self.is_grad else FLOPS_PER_PAIR)[w["kernel"]](k)
+
+        x = self.x_cpu.to(device)
+        rhs = self.rhs_cpu.to(device)
+        self.params = self.params_cpu.to(device)
+        start, end = self.start_cpu.to(device), self.end_cpu.to(device)
+        # batch items share x, rhs and the pattern (stride-0 views), as KernelMatmulLinearOperator passes them
+        xb = x.expand(*bshape, n)
+        rhsb = rhs.expand(*bshape, n, k)
+        startb = start.expand(*bshape, row_blocks)
+        endb = end.expand(*bshape, row_blocks)
+        if name == "c3_rhs_grad":
+            # d/d rhs of sum(grad_out * (K @ rhs)) = K^T @ grad_out: the forward kernel on the
+            # (symmetric) pattern with a per-batch-item grad_out in place of rhs
+            g2 = torch.Generator().manual_seed(w["seed"] + 60)
+            rhsb = torch.randn(*bshape, n, k, generator=g2).to(device)
+        self.args = (xb, xb, rhsb, self.params, startb, endb)
+        defines = MatmulSingleConfiguration(w["kernel"]).make_config(self.args)
+        if variant != "auto":
+            defines["MATMUL_VARIANT"] = variant
+        if rows_per_wave:
+            defines["MATMUL_ROWS_PER_WAVE"] = rows_per_wave
+        if col_splits:
+            defines["MATMUL_COL_BLOCKS"] = col_splits
+        if not tail_balance:
+            defines["MATMUL_TAIL_BALANCE"] = 0
+        self.op = load_native("matmul", defines)
+        self.kernel = self.op.describe(*self.args)
+        if self.is_grad:
+            g2 = torch.Generator().manual_seed(w["seed"] + 50)
+            left = torch.randn(n, k, generator=g2).to(device).expand(*bshape, n, k)
+            self.args = (xb, xb, left, rhsb, self.params, startb, endb)
+            self.op = load_native("bilinear_derivative",
+                                  BilinearDerivativeConfiguration(w["kernel"]).make_config(self.args))
+            self.kernel = self.op.describe(*self.args)
+
+    def call(self):
+        return self.op.call(*self.args)
+
+    def measure(self, steps, warmup):
+        """(wall ms per step, mean and median kernel ms by events on the launch stream, last output)."""
+        import torch
+
+        out = None
+        for _ in range(warmup):
+            out = self.call()
+        torch.cuda.synchronize()
+        events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+                  for _ in range(steps)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for e0, e1 in events:
+            e0.record()
+            out = self.call()
+            e1.record()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        kernel_ms = sorted(e0.elapsed_time(e1) for e0, e1 in events)
+        return (t1 - t0) * 1e3 / steps, sum(kernel_ms) / len(kernel_ms), kernel_ms[len(kernel_ms) // 2], out
+
+    def summary(self, steps, warmup):
+        wall_ms, kernel_ms, _, _ = self.measure(steps, warmup)
+        tflops = self.pairs * self.flops_per_pair / (kernel_ms * 1e-3) / 1e12
+        return {
+            "workload": self.w["label"],
+            "kernel": self.kernel,
+            "pairs_per_call": self.pairs,
+            "flops_per_pair": self.flops_per_pair,
+            "kernel_ms": kernel_ms,
+            "wall_ms_per_call": wall_ms,
+            "pairs_per_s_kernel": self.pairs / (kernel_ms * 1e-3),
+            "pairs_per_s_wall": self.pairs / (wall_ms * 1e-3),
+            "frac_of_fp32_peak": tflops / PEAK_FP32_TFLOPS,
+        }
+
+
+def full_output_fp64(p: Prepared):
+    """float64 K @ rhs over the whole pattern of a forward workload, one row block at a time."""
+    import numpy as np
+
+    from oracle import kernels as oracle
+
+    x = p.x_cpu.numpy()
+    rhs = p.rhs_cpu.double().numpy()
+    params = p.params_cpu.numpy().reshape(-1, p.params_cpu.shape[-1])
+    start, end = p.start_cpu.numpy(), p.end_cpu.numpy()
+    n, nb = x.shape[0], params.shape[0]
+    out = np.zeros((nb, n, rhs.shape[-1]))
+    for blk in range(len(start)):
+        r0, r1 = blk * 128, min(blk * 128 + 128, n)
+        s, e = int(start[blk]), min(int(end[blk]), n)
+        if s < e:
+            kb = oracle.kernel_matrix(p.w["kernel"], np.broadcast_to(x[r0:r1], (nb, r1 - r0)),
+                                      np.broadcast_to(x[s:e], (nb, e - s)), params)
+            out[:, r0:r1] = kb @ rhs[s:e]
+    return out
 
 
 def main() -> int:
@@ -84,7 +216,9 @@ def main() -> int:
     ap.add_argument("--col-splits", type=int, default=0)
     ap.add_argument("--batch", type=int, default=None, help="override the number of batch items")
     ap.add_argument("--no-tail-balance", action="store_true")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-cpu-baseline", action="store_true",
+                    help="skip the host-side legs: the CPU baseline and the float64 error figures")
+    ap.add_argument("--no-configs", action="store_true", help="skip the other benchmark configurations")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB elementwise add-scalar (a copy-like kernel of known traffic "
                          "against which FETCH_SIZE / WRITE_SIZE counters are scaled)")
@@ -99,9 +233,6 @@ def main() -> int:
     import torch
 
     from kernel_matmul_amd import _native
-    from kernel_matmul_amd.compile import load_native
-    from kernel_matmul_amd.configurations import MatmulSingleConfiguration
-    from kernel_matmul_amd.ranges import make_ranges
 
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
@@ -109,49 +240,13 @@ def main() -> int:
     _native.load_library()  # fail loudly if the HIP library is missing
     device = torch.device("cuda:0")
 
-    w, x_cpu, params_cpu, rhs_cpu, cutoff = make_workload(args.workload, args.batch)
-    n, k, batch = w["n"], w["k"], w["batch"]
-    bshape = (batch,) if batch else ()
-    start_cpu, end_cpu = make_ranges(cutoff, x_cpu)  # symmetric pattern, block 128
-    row_blocks = start_cpu.shape[-1]
-    rows_in_block = torch.clamp(n - 128 * torch.arange(row_blocks), max=128)
-    pairs_per_item = int((rows_in_block * (end_cpu - start_cpu)).sum())
-    pairs = pairs_per_item * max(batch, 1)
-    is_grad = w.get("op") == "param_grad"
-    flops_per_pair = (GRAD_FLOPS_PER_PAIR if is_grad else FLOPS_PER_PAIR)[w["kernel"]](k)
-
-    x = x_cpu.to(device)
-    rhs = rhs_cpu.to(device)
-    params = params_cpu.to(device)
-    start, end = start_cpu.to(device), end_cpu.to(device)
-    # batch items share x, rhs and the pattern (stride-0 views), as KernelMatmulLinearOperator passes them
-    xb = x.expand(*bshape, n)
-    rhsb = rhs.expand(*bshape, n, k)
-    startb = start.expand(*bshape, row_blocks)
-    endb = end.expand(*bshape, row_blocks)
-    op_args = (xb, xb, rhsb, params, startb, endb)
-
-    defines = MatmulSingleConfiguration(w["kernel"]).make_config(op_args)
-    if args.variant != "auto":
-        defines["MATMUL_VARIANT"] = args.variant
-    if args.rows_per_wave:
-        defines["MATMUL_ROWS_PER_WAVE"] = args.rows_per_wave
-    if args.col_splits:
-        defines["MATMUL_COL_BLOCKS"] = args.col_splits
-    if args.no_tail_balance:
-        defines["MATMUL_TAIL_BALANCE"] = 0
-    op = load_native("matmul", defines)
-    if is_grad:
-        from kernel_matmul_amd.configurations import BilinearDerivativeConfiguration
-
-        g2 = torch.Generator().manual_seed(w["seed"] + 50)
-        left = torch.randn(n, k, generator=g2).to(device).expand(*bshape, n, k)
-        op_args = (xb, xb, left, rhsb, params, startb, endb)
-        op = load_native("bilinear_derivative",
-                         BilinearDerivativeConfiguration(w["kernel"]).make_config(op_args))
+    main_run = Prepared(args.workload, device, args.batch, args.variant, args.rows_per_wave, args.col_splits,
+                        not args.no_tail_balance)
+    w = main_run.w
+    n, batch = w["n"], w["batch"]
 
     for _ in range(args.warmup):
-        out = op.call(*op_args)
+        out = main_run.call()
     torch.cuda.synchronize()
     if args.calibrate_copy:
         src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device=device)
@@ -162,42 +257,13 @@ def main() -> int:
         del src, dst
 
     # Whole-step wall time and, on the launch stream, per-launch event time of the kernel.
-    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
-              for _ in range(args.steps)]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for e0, e1 in events:
-        e0.record()
-        out = op.call(*op_args)
-        e1.record()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
-    kernel_ms = sorted(e0.elapsed_time(e1) for e0, e1 in events)
-    kernel_ms_avg = sum(kernel_ms) / len(kernel_ms)
-    kernel_ms_med = kernel_ms[len(kernel_ms) // 2]
-
+    ms_per_step, kernel_ms_avg, kernel_ms_med, out = main_run.measure(args.steps, 0)
+    pairs, flops_per_pair = main_run.pairs, main_run.flops_per_pair
     value = pairs / (ms_per_step * 1e-3)
     achieved_tflops = pairs * flops_per_pair / (kernel_ms_avg * 1e-3) / 1e12
 
-    # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
-    # profiles/fwd_table_f16_headline_counters.md (only measured for the default headline run).
-    traffic = None
-    if args.workload == "headline" and args.batch is None and args.variant in ("auto", "mfma_f16"):
-        traffic = MEASURED_TRAFFIC_BYTES["headline"]
-
-    # Kernel the launch table picks for this workload / variant: column tables (spectral in
-    # phase-split form) for rbf / spectral with at most 16 rhs columns, the shared-operand kernel
-    # for large rbf / locally periodic problems, direct evaluation otherwise.
-    row_block_items = ((n + 127) // 128) * max(batch, 1)
-    table = w["kernel"] in ("spectral", "rbf") and k <= 16
-    shared = w["kernel"] != "spectral" and k <= 16 and row_block_items >= 4096
-    auto_kernel = "km::fwd_block" if shared else ("km::fwd_table_f16" if table else "km::fwd_mfma_f16")
-    kernel_name = "km::param_grad_partial" if is_grad else {
-        "auto": auto_kernel,
-        "mfma_f16": "km::fwd_table_f16" if table else "km::fwd_mfma_f16",
-        "mfma_f16_direct": "km::fwd_mfma_f16", "block": "km::fwd_block",
-        "mfma_f32": "km::fwd_mfma_f32", "valu": "km::fwd_valu"}[args.variant]
+    default_run = args.workload == "headline" and args.batch is None and args.variant in ("auto", "mfma_f16")
+    traffic = MEASURED_TRAFFIC_BYTES["headline"] if default_run else None
 
     result = {
         "metric": "kernel-pair evaluations/s (sparse spectral K@rhs, n=100k, k=16, 1 MI355X)",
@@ -210,38 +276,84 @@ def main() -> int:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        "dtype": "f32 in/out, K evaluated in f32 on the VALU; contraction: split-fp16 MFMA (hi+lo, 22 bits per "
+                 "factor) with f32 accumulation" if args.variant in ("auto", "mfma_f16", "mfma_f16_direct", "block")
+                 else "f32",
         "data": "synthetic",
         "config": {
             "workload": w["label"],
             "pairs_per_step": pairs,
             "flops_per_pair": flops_per_pair,
-            "variant": op.defines.get("MATMUL_VARIANT", "auto (split-fp16 MFMA)"),
+            "variant": main_run.op.defines.get("MATMUL_VARIANT", "auto"),
             "seed": w["seed"],
         },
         "roofline": {
-            "bound": "mfma",
-            "kernel": kernel_name,
+            "bound": "valu",
+            "kernel": main_run.kernel,
             "achieved": achieved_tflops,
             "peak": PEAK_FP32_TFLOPS,
             "unit": "TFLOP/s",
             "frac": achieved_tflops / PEAK_FP32_TFLOPS,
             "traffic": traffic,
+            "traffic_source": TRAFFIC_SOURCE + " (offline counter run, not measured by this run)" if traffic else None,
             "kernel_ms_avg": kernel_ms_avg,
             "kernel_ms_median": kernel_ms_med,
             "pairs_per_s_kernel": pairs / (kernel_ms_avg * 1e-3),
-            "note": "priced against the fp32 peak (157.3 TFLOP/s vector == fp32 MFMA): K is evaluated in "
-                    "fp32 on the VALU, the contraction runs as split-fp16 MFMAs with fp32 accumulation; "
-                    "flops = pairs * (8 + 2k), one transcendental counted as 1",
+            "note": "bound by VALU issue (kernel evaluation in fp32 + hi/lo split + MFMA issue), priced against "
+                    "the fp32 peak (157.3 TFLOP/s vector == fp32 MFMA); flops = pairs * (8 + 2k), one "
+                    "transcendental counted as 1.  The contraction itself runs as split-fp16 MFMAs, so frac is "
+                    "a figure of merit against the fp32 roofline, not a utilisation of one pipe",
         },
     }
 
-    if not args.no_cpu_baseline and not is_grad:
+    if default_run:
+        # The same workload with the contraction as a true fp32 MFMA (v_mfma_f32_16x16x4_f32).
+        f32_run = Prepared("headline", device, variant="mfma_f32")
+        _, f32_ms, _, f32_out = f32_run.measure(max(args.steps // 2, 5), 2)
+        result["roofline"]["fp32_mfma_variant"] = {
+            "kernel": f32_run.kernel,
+            "kernel_ms": f32_ms,
+            "frac": pairs * flops_per_pair / (f32_ms * 1e-3) / 1e12 / PEAK_FP32_TFLOPS,
+        }
+    else:
+        f32_out = None
+
+    if not args.no_configs and default_run:
+        configs = {}
+        for name in ("c1", "c2", "c3", "c3_rhs_grad", "c4", "c5", "ref_example"):
+            run = Prepared(name, device)
+            configs[name] = run.summary(steps=20 if name != "c5" else 10, warmup=3)
+            del run
+            torch.cuda.empty_cache()
+        result["configs"] = configs
+
+    if not args.no_cpu_baseline and not main_run.is_grad:
+        import numpy as np
+
         from oracle import dense_cpu
 
+        if default_run:
+            # Error of both contractions over the whole output against float64.
+            expected = full_output_fp64(main_run)
+            scale = np.abs(expected).max()
+            errors = {}
+            for label, tensor in (("auto", out), ("mfma_f32", f32_out)):
+                err = np.abs(tensor.cpu().double().numpy() - expected)
+                errors[label] = {
+                    "max_abs": float(err.max()),
+                    "max_abs_over_output_scale": float(err.max() / scale),
+                    "max_rel_where_abs_expected_ge_1e-3": float((err / np.maximum(np.abs(expected), 1e-3)).max()),
+                    "rms": float(np.sqrt((err * err).mean())),
+                }
+            errors["output_scale_max_abs"] = float(scale)
+            errors["tolerance"] = "rtol 1e-4 / atol 1e-5 (tests), both variants within it"
+            result["roofline"]["error_vs_fp64"] = errors
+            del expected
+
+        x_cpu, rhs_cpu, params_cpu = main_run.x_cpu, main_run.rhs_cpu, main_run.params_cpu
         p0 = params_cpu[0] if batch else params_cpu
         sec, in_band, dense_pairs, slabs, rows = dense_cpu.time_masked_matmul(
-            w["kernel"], x_cpu, x_cpu, rhs_cpu, p0, start_cpu, end_cpu, args.cpu_seconds)
+            w["kernel"], x_cpu, x_cpu, rhs_cpu, p0, main_run.start_cpu, main_run.end_cpu, args.cpu_seconds)
         got = (out[0] if batch else out)[: rows.shape[0]].cpu()
         err = (got - rows).abs().max().item()
         result["cpu_baseline"] = {

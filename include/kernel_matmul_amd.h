@@ -118,6 +118,14 @@ int km_matmul(int kernel_type, int batch_rank, const int64_t* batch_sizes, int64
               const int64_t* start_strides, const int32_t* end, const int64_t* end_strides,
               float* out, const km_launch_options* options, void* stream);
 
+/* Which ahead-of-time kernel and decomposition km_matmul would pick for a problem of this
+ * size (host only; nothing is launched).  Writes a short description such as
+ * "km::fwd_table_f16<spectral, G=1, R=8>: 128 rows per wavefront, ..." into `text`.
+ * Stands in for the reference's autotune report (kernel_matmul/native_function.py:56-69,
+ * which prints the winning define set). */
+int km_matmul_describe(int kernel_type, int64_t num_batches, int64_t m, int64_t n, int64_t k,
+                       const km_launch_options* options, char* text, size_t text_bytes);
+
 /* ------------------------------------------------------------------------------------
  * Hyper-parameter gradient of a bilinear form through the masked kernel matrix:
  *   grad[b,p] = d/d params[b,p]  sum_{(i,j) in mask} (sum_c left[b,i,c] right[b,j,c]) K[b,i,j]

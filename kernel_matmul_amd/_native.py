@@ -83,6 +83,9 @@ def load_library():
         + tensor * 6
         + [_vp, ctypes.POINTER(LaunchOptions), _vp]
     )
+    lib.km_matmul_describe.restype = ctypes.c_int
+    lib.km_matmul_describe.argtypes = [ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                                       ctypes.c_int64, _vp, ctypes.c_char_p, ctypes.c_size_t]
     lib.km_param_grad_workspace_size.restype = ctypes.c_size_t
     lib.km_param_grad_workspace_size.argtypes = [ctypes.c_int, ctypes.c_int, _i64p, ctypes.c_int64,
                                                  ctypes.c_int64, ctypes.c_int64]
@@ -302,6 +305,18 @@ def matmul(kernel_type: str, x1: Tensor, x2: Tensor, rhs: Tensor, params: Tensor
     if status != 0:
         _raise(load_library(), status)
     return out
+
+
+def describe_matmul(kernel_type: str, num_batches: int, m: int, n: int, k: int,
+                    options: LaunchOptions | None = None) -> str:
+    """Kernel and decomposition the launch table picks for this problem (C ABI: km_matmul_describe)."""
+    lib = load_library()
+    text = ctypes.create_string_buffer(256)
+    status = lib.km_matmul_describe(_kernel_id(kernel_type), num_batches, m, n, k,
+                                    ctypes.byref(options) if options is not None else None, text, 256)
+    if status != 0:
+        _raise(lib, status)
+    return text.value.decode()
 
 
 def param_grad(kernel_type: str, x1: Tensor, x2: Tensor, left: Tensor, right: Tensor,

@@ -115,6 +115,20 @@ class NativeModule:
             options.rows_per_wave = int(rows)
         return options
 
+    def describe(self, *args) -> str:
+        """Which kernel and decomposition ``call(*args)`` runs (matmul only; nothing is launched)."""
+        if self.op != "matmul":
+            return {"matmul_bwd": "km::param_grad_partial + km::param_grad_reduce",
+                    "bilinear_derivative": "km::param_grad_partial + km::param_grad_reduce",
+                    "index": "km::index_kernel", "index_bwd": "km::index_bwd_terms + reduce",
+                    "dense": "km::dense_kernel", "dense_bwd": "km::dense_bwd_partial + reduce"}[self.op]
+        x1, x2, rhs = args[0], args[1], args[2]
+        batches = 1
+        for size in x1.shape[:-1]:
+            batches *= size
+        return _native.describe_matmul(self.kernel_type, batches, x1.shape[-1], x2.shape[-1], rhs.shape[-1],
+                                       self._options)
+
     def _check_batch_dim(self, x1) -> None:
         declared = self.defines.get("BATCH_DIM")
         if declared is not None and declared != x1.dim() - 1:

@@ -369,6 +369,54 @@ int km_matmul(int kernel_type, int batch_rank, const int64_t* batch_sizes, int64
     return err == hipSuccess ? KM_OK : fail_hip(op, err);
 }
 
+int km_matmul_describe(int kernel_type, int64_t num_batches, int64_t m, int64_t n, int64_t k,
+                       const km_launch_options* options, char* text, size_t text_bytes) {
+    const char* op = "km_matmul_describe";
+    if (km_num_params(kernel_type) < 0) {
+        return fail(KM_ERR_UNSUPPORTED, "%s: unknown kernel type %d", op, kernel_type);
+    }
+    if (num_batches < 0 || m < 0 || n < 0 || k < 0 || text == nullptr || text_bytes == 0) {
+        return fail(KM_ERR_INVALID_ARGUMENT, "%s: invalid argument", op);
+    }
+    MatmulProblem p;
+    memset(&p, 0, sizeof(p));
+    p.kernel_type = kernel_type;
+    p.num_batches = num_batches;
+    p.m = m;
+    p.n = n;
+    p.k = k;
+    MatmulPlan plan;
+    if (int rc = make_plan(p, options, &plan)) return rc;
+    static const char* const kernels[] = {"rbf", "spectral", "locally_periodic"};
+    const char* kt = kernels[kernel_type];
+    const long long row_blocks = (m + KM_BLOCK_SIZE - 1) / KM_BLOCK_SIZE;
+    const int G = plan.k_chunk / 16;
+    switch (plan.variant) {
+        case KM_VARIANT_VALU:
+            snprintf(text, text_bytes, "km::fwd_valu<%s, KC=%d>: 128 rows per workgroup, %lld workgroups", kt,
+                     plan.k_chunk, row_blocks * num_batches * ((k + plan.k_chunk - 1) / plan.k_chunk));
+            break;
+        case KM_VARIANT_BLOCK:
+            snprintf(text, text_bytes,
+                     "km::fwd_block<%s, phase_split=%d, G=%d>: 4 wavefronts per 4 row blocks, rhs operand shared in LDS",
+                     kt, plan.phase_split, G);
+            break;
+        default: {
+            const char* name = plan.variant == KM_VARIANT_MFMA_F32
+                                   ? "km::fwd_mfma_f32"
+                                   : (plan.variant == KM_VARIANT_MFMA_F16 ? "km::fwd_table_f16" : "km::fwd_mfma_f16");
+            snprintf(text, text_bytes, "%s<%s, G=%d, R=%d>: %d rows per wavefront, %d wavefront(s) per row range%s",
+                     name, kt, G, plan.row_groups, 16 * plan.row_groups, plan.col_splits,
+                     plan.tail_balance && plan.row_groups == 8 && plan.col_splits == 1 &&
+                             plan.variant != KM_VARIANT_MFMA_F32
+                         ? ", tail items cut into 16-row pieces"
+                         : "");
+            break;
+        }
+    }
+    return KM_OK;
+}
+
 // ---------------------------------------------------------------------------------------
 // param_grad (matmul_bwd and bilinear_derivative)
 // ---------------------------------------------------------------------------------------
