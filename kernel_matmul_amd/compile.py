@@ -110,6 +110,8 @@ class NativeModule:
                                "block": 5}[variant]
         if self.defines.get("MATMUL_TAIL_BALANCE") == 0:
             options.reserved = 1
+        elif self.defines.get("MATMUL_GROUP_TAIL") is not None:
+            options.reserved = 2 + int(self.defines["MATMUL_GROUP_TAIL"])
         rows = self.defines.get("MATMUL_ROWS_PER_WAVE")
         if rows is not None:
             options.rows_per_wave = int(rows)

@@ -89,6 +89,10 @@ static const long long BLOCK_VARIANT_MIN_ITEMS = 4096;
 static int make_plan(const MatmulProblem& p, const km_launch_options* opt, MatmulPlan* plan) {
     int variant = opt ? opt->variant : KM_VARIANT_AUTO;
     plan->phase_split = 0;
+    plan->group_tail = -1;
+    if (opt && opt->reserved >= 2) {
+        plan->group_tail = opt->reserved - 2;  // measurements: grouped launch with this many split items per XCD
+    }
     if (variant == KM_VARIANT_AUTO) {
         // Measured on gfx950 (n = 1e5 ... 1e6, batch 2 ... 8): with up to 16 rhs columns and enough
         // row blocks to fill the device several times, sharing the rhs operand between four row
@@ -181,6 +185,20 @@ static int make_plan(const MatmulProblem& p, const km_launch_options* opt, Matmu
     plan->row_groups = R;
     plan->col_splits = S;
     plan->tail_balance = !(opt && opt->reserved == 1);  // reserved = 1 switches it off (measurements)
+    // Table kernel with one wavefront per 128-row item and enough items to run several rounds
+    // per SIMD: grouped launch (workgroups of 4 wavefronts) whose last items are split by
+    // columns.  Measured at n = 1e5, k = 16 (782 items per XCD at batch 8): 12-19 % of an XCD's
+    // items split this way is best (112.7 us against 118.7 us with 16-row tail pieces; batch 64:
+    // 751 against 773 us); more than a third of a round of wavefronts (128 items) gains nothing.
+    if (table && R == 8 && S == 1 && plan->tail_balance && plan->group_tail < 0) {
+        const long long per_xcd = (row_blocks * p.num_batches + KM_NUM_XCD - 1) / KM_NUM_XCD;
+        if (per_xcd >= 2 * 128) {
+            plan->group_tail = per_xcd / 7 < 128 ? per_xcd / 7 : 128;
+        }
+    }
+    if (!(table && R == 8 && S == 1)) {
+        plan->group_tail = -1;
+    }
     return KM_OK;
 }
 
@@ -405,10 +423,18 @@ int km_matmul_describe(int kernel_type, int64_t num_batches, int64_t m, int64_t 
             const char* name = plan.variant == KM_VARIANT_MFMA_F32
                                    ? "km::fwd_mfma_f32"
                                    : (plan.variant == KM_VARIANT_MFMA_F16 ? "km::fwd_table_f16" : "km::fwd_mfma_f16");
+            if (plan.variant == KM_VARIANT_MFMA_F16 && plan.group_tail >= 0) {
+                snprintf(text, text_bytes,
+                         "km::fwd_table_f16_grouped<%s>: 128 rows per wavefront, 4 wavefronts per workgroup, the "
+                         "last %lld items of each XCD split by columns over a workgroup",
+                         kt, plan.group_tail);
+                break;
+            }
             snprintf(text, text_bytes, "%s<%s, G=%d, R=%d>: %d rows per wavefront, %d wavefront(s) per row range%s",
                      name, kt, G, plan.row_groups, 16 * plan.row_groups, plan.col_splits,
                      plan.tail_balance && plan.row_groups == 8 && plan.col_splits == 1 &&
-                             plan.variant != KM_VARIANT_MFMA_F32
+                             plan.variant == KM_VARIANT_MFMA_F16_DIRECT &&
+                             row_blocks * num_batches >= 2 * 128 * KM_NUM_XCD
                          ? ", tail items cut into 16-row pieces"
                          : "");
             break;

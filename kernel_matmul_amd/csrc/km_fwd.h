@@ -24,7 +24,8 @@ struct FwdArgs {
     long long items_per_xcd;
     int m, n, k;
     int chunks_per_block;    // 128 / rows per workgroup
-    int tail_items;          // per XCD: row-block items at the end that are split 8 ways by rows
+    int tail_items;          // per XCD: row-block items at the end that are dispatched last in pieces
+                             // (direct kernel: 8 pieces of 16 rows; grouped table kernel: 4 column shares)
     const float* x1;
     const float* x2;
     const float* rhs;

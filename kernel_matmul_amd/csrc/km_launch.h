@@ -45,6 +45,8 @@ struct MatmulPlan {
     int col_splits;  // MFMA: wavefronts per workgroup sharing one column range (1, 2, 4, 8)
     int tail_balance;  // split-fp16 kernels: cut the uneven remainder into 16-row pieces
     int phase_split;   // KM_VARIANT_BLOCK: spectral kernel in phase-split form
+    long long group_tail;  // table kernel: >= 0 selects the grouped launch (workgroups of 4 wavefronts) with
+                           // this many items per XCD split by columns at the end; < 0: one wavefront per workgroup
 };
 
 hipError_t launch_matmul(const MatmulProblem& p, const MatmulPlan& plan, hipStream_t stream);

@@ -666,9 +666,12 @@ __device__ __forceinline__ void rhs_load(const FwdArgs& a, const WaveView& w, in
     }
 }
 
+// S wavefronts (this one is number `wave` of them) share the row range and split its columns;
+// `slot` is the wavefront's table area in LDS.  With `overlay` the cross-wavefront reduction
+// buffer lies over the table areas instead of behind them.
 template <int KT, int G, int R>
 __device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds, const WaveView& wv,
-                                                   int row0) {
+                                                   int row0, int S, int wave, int slot, bool overlay) {
     static_assert(KT == KM_KERNEL_SPECTRAL || KT == KM_KERNEL_RBF, "table kernel: rbf or spectral");
     constexpr bool PHASE = KT == KM_KERNEL_SPECTRAL;
     // Accumulator groups; phase-split: [cos part of g = 0..G), sin part of g = 0..G)].
@@ -678,8 +681,6 @@ __device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds,
     constexpr int KS = KM_TABLE_KSCALE_LOG2;
 
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int S = blockDim.x >> 6;
     const int li = lane & 15;
     const int kk = lane >> 4;
     const int kbase = blockIdx.y * (16 * G);
@@ -731,12 +732,12 @@ __device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds,
     // Per-wavefront table of the current chunk: x2, b = (x2 - r) s with r the x2 value in the
     // middle of each group of 8 columns, the two column factors of the rhs operand (cos B and
     // sin B, times 2^(-b^2) in the separable form; rbf: the first alone), and the r's.
-    float* tab_x2 = lds + (size_t)wave * KM_PHASE_TABLE_FLOATS;
+    float* tab_x2 = lds + (size_t)slot * KM_PHASE_TABLE_FLOATS;
     float* tab_b = tab_x2 + CH;
     float* tab_cos = tab_b + CH;
     float* tab_sin = tab_cos + CH;
     float* tab_ref = tab_sin + CH;
-    float* reduce_buffer = lds + (size_t)S * KM_PHASE_TABLE_FLOATS;
+    float* reduce_buffer = overlay ? lds : lds + (size_t)S * KM_PHASE_TABLE_FLOATS;
 
     float row_lo = __builtin_inff(), row_hi = -__builtin_inff();
     bool row_nan = false;
@@ -926,6 +927,9 @@ __device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds,
     if (S == 1) {
         store_direct<G, R>(res, lane, out, row0, kbase, a.m, a.k);
     } else {
+        if (overlay) {
+            __syncthreads();  // every wavefront is done with its table
+        }
         reduce_and_store<G, R>(res, reduce_buffer, S, wave, lane, out, row0, kbase, a.m, a.k);
     }
 }
@@ -933,20 +937,55 @@ __device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds,
 template <int KT, int G, int R>
 __global__ void __launch_bounds__(512, 3) fwd_table_f16(const FwdArgs a) {
     extern __shared__ float lds[];
-    const ItemRef it = decode_item(a);
-    if (!it.valid) {
+    const long long item = xcd_item(blockIdx.x, a.items_per_xcd);
+    if (item >= a.total_items) {
         return;
     }
     int chunk_in_block;
-    if constexpr (R == 8) {
-        if (it.small) {
-            const WaveView w = wave_view(a, it.item, 1, &chunk_in_block);
-            fwd_table_f16_body<KT, G, 1>(a, lds, w, w.row_block * KM_BLOCK_SIZE + 16 * it.piece);
+    const WaveView w = wave_view(a, item, a.chunks_per_block, &chunk_in_block);
+    // (the wavefront index is wave-uniform by construction; saying so keeps what is derived from
+    // it in scalar registers)
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    fwd_table_f16_body<KT, G, R>(a, lds, w, w.row_block * KM_BLOCK_SIZE + chunk_in_block * (16 * R),
+                                 blockDim.x >> 6, wave, wave, false);
+}
+
+// Grouped launch of the table kernel for large problems (one wavefront per 128-row item, up to
+// 16 rhs columns): workgroups of 4 wavefronts.  The first items of every XCD go one per
+// wavefront, four to a workgroup; its last `tail_items` items are dispatched last, one per
+// workgroup, with the four wavefronts splitting the item's column range (no repeated work) and
+// adding their shares in a fixed order through LDS.  These quarter-length pieces fill the SIMDs
+// while the last full items finish.
+#define KM_GROUP_WAVES 4
+
+template <int KT>
+__global__ void __launch_bounds__(64 * KM_GROUP_WAVES, 3) fwd_table_f16_grouped(const FwdArgs a) {
+    extern __shared__ float lds[];
+    // The wavefront index is wave-uniform by construction; saying so keeps the item and
+    // everything derived from it (pointers, ranges, parameters) in scalar registers.
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const unsigned xcd = blockIdx.x % KM_NUM_XCD;
+    const long long slot = blockIdx.x / KM_NUM_XCD;
+    const long long main_items = a.items_per_xcd - a.tail_items;
+    const long long main_groups = (main_items + KM_GROUP_WAVES - 1) / KM_GROUP_WAVES;
+    const bool split = slot >= main_groups;
+    long long local;
+    if (!split) {
+        local = slot * KM_GROUP_WAVES + wave;
+        if (local >= main_items) {
             return;
         }
+    } else {
+        local = main_items + (slot - main_groups);
     }
-    const WaveView w = wave_view(a, it.item, a.chunks_per_block, &chunk_in_block);
-    fwd_table_f16_body<KT, G, R>(a, lds, w, w.row_block * KM_BLOCK_SIZE + chunk_in_block * (16 * R));
+    const long long item = (long long)xcd * a.items_per_xcd + local;
+    if (item >= a.total_items) {
+        return;  // uniform for the workgroup of a split item
+    }
+    int unused;
+    const WaveView w = wave_view(a, item, 1, &unused);
+    fwd_table_f16_body<KT, 1, 8>(a, lds, w, w.row_block * KM_BLOCK_SIZE, split ? KM_GROUP_WAVES : 1,
+                                 split ? wave : 0, wave, true);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -1124,11 +1163,10 @@ hipError_t launch_matmul(const MatmulProblem& p, const MatmulPlan& plan, hipStre
     a.tail_items = 0;
     unsigned grid_x = (unsigned)(a.items_per_xcd * KM_NUM_XCD);
     const unsigned grid_y = (unsigned)((p.k + plan.k_chunk - 1) / plan.k_chunk);
-    // Tail balancing (split-fp16 kernels, one wavefront per 128-row block): whatever does not
-    // fill all 128 SIMDs of an XCD evenly is cut into 16-row pieces and dispatched last.
-    const bool f16 = plan.variant == KM_VARIANT_MFMA_F16 || plan.variant == KM_VARIANT_MFMA_F16_DIRECT;
-    if (f16 && plan.row_groups == 8 && plan.col_splits == 1 && plan.tail_balance &&
-        a.items_per_xcd >= 2 * 128) {
+    // Tail balancing (direct split-fp16 kernel, one wavefront per 128-row block): whatever does
+    // not fill all 128 SIMDs of an XCD evenly is cut into 16-row pieces and dispatched last.
+    if (plan.variant == KM_VARIANT_MFMA_F16_DIRECT && plan.row_groups == 8 && plan.col_splits == 1 &&
+        plan.tail_balance && a.items_per_xcd >= 2 * 128) {
         a.tail_items = (int)(a.items_per_xcd % 128);
         grid_x = (unsigned)((a.items_per_xcd - a.tail_items + 8LL * a.tail_items) * KM_NUM_XCD);
     }
@@ -1139,6 +1177,23 @@ hipError_t launch_matmul(const MatmulProblem& p, const MatmulPlan& plan, hipStre
             case KM_KERNEL_SPECTRAL: return launch_valu<KM_KERNEL_SPECTRAL>(a, plan.k_chunk, grid_x, grid_y, stream);
             default: return launch_valu<KM_KERNEL_LOCALLY_PERIODIC>(a, plan.k_chunk, grid_x, grid_y, stream);
         }
+    }
+    if (plan.variant == KM_VARIANT_MFMA_F16 && plan.group_tail >= 0 && plan.row_groups == 8 &&
+        plan.col_splits == 1 && plan.k_chunk == 16 && p.kernel_type != KM_KERNEL_LOCALLY_PERIODIC) {
+        a.tail_items = (int)(plan.group_tail < a.items_per_xcd ? plan.group_tail : a.items_per_xcd);
+        const long long main_groups = (a.items_per_xcd - a.tail_items + KM_GROUP_WAVES - 1) / KM_GROUP_WAVES;
+        const unsigned gx = (unsigned)((main_groups + a.tail_items) * KM_NUM_XCD);
+        const size_t table = (size_t)KM_GROUP_WAVES * KM_PHASE_TABLE_FLOATS * sizeof(float);
+        static_assert(KM_GROUP_WAVES * 8 * 4 * 64 <= KM_GROUP_WAVES * KM_PHASE_TABLE_FLOATS,
+                      "the reduction buffer of a split item must fit over the tables");
+        if (p.kernel_type == KM_KERNEL_SPECTRAL) {
+            hipLaunchKernelGGL((fwd_table_f16_grouped<KM_KERNEL_SPECTRAL>), dim3(gx, grid_y, 1),
+                               dim3(64 * KM_GROUP_WAVES, 1, 1), table, stream, a);
+        } else {
+            hipLaunchKernelGGL((fwd_table_f16_grouped<KM_KERNEL_RBF>), dim3(gx, grid_y, 1),
+                               dim3(64 * KM_GROUP_WAVES, 1, 1), table, stream, a);
+        }
+        return hipGetLastError();
     }
     const int G = plan.k_chunk / 16;
     switch (p.kernel_type) {

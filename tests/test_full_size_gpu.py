@@ -157,6 +157,25 @@ def test_forward_every_row_block_against_oracle(name, variant):
     assert np.all(err <= tol), (name, variant, worst, err[worst], expected[worst])
 
 
+@pytest.mark.parametrize("name,group_tail", [("headline", 0), ("headline", 97), ("headline", 10_000),
+                                             ("c2", 5), ("c3_rbf", 3)])
+def test_forward_grouped_launch_against_oracle(name, group_tail):
+    """Workgroups of four wavefronts: full items one per wavefront, the last `group_tail` items of
+    every XCD split by columns between the four wavefronts of a workgroup (fixed-order sum)."""
+    kernel, n, batch, k, a, h = _build(name)
+    op_args = (a["x"], a["x"], a["rhs"], a["params"], a["start"], a["end"])
+    defines = MatmulSingleConfiguration(kernel).make_config(op_args)
+    defines["MATMUL_VARIANT"] = "mfma_f16"
+    defines["MATMUL_ROWS_PER_WAVE"] = 128
+    defines["MATMUL_GROUP_TAIL"] = group_tail
+    out = load_native("matmul", defines).call(*op_args)
+    again = load_native("matmul", defines).call(*op_args)
+    assert torch.equal(out, again)  # fixed reduction order: reproducible
+    expected = _forward_oracle(name, kernel, h)
+    err = np.abs(out.cpu().double().numpy() - expected)
+    assert np.all(err <= 1e-5 + 1e-4 * np.abs(expected)), (name, group_tail, err.max())
+
+
 def test_split_fp16_error_against_fp32_mfma_on_headline():
     """How much accuracy the split-fp16 contraction (the default) trades against the fp32 MFMA
     contraction, over the full headline output, each against the float64 oracle.  Both must
