@@ -448,13 +448,16 @@ int km_matmul_describe(int kernel_type, int64_t num_batches, int64_t m, int64_t 
 // ---------------------------------------------------------------------------------------
 size_t km_param_grad_workspace_size(int kernel_type, int batch_rank, const int64_t* batch_sizes,
                                     int64_t m, int64_t n, int64_t c) {
-    (void)c;
     long long nb = 0;
     if (check_common("km_param_grad_workspace_size", kernel_type, batch_rank, batch_sizes, m, n, &nb)) {
         return 0;
     }
     if (nb == 0 || m == 0) return 0;
-    return (size_t)nb * (size_t)param_grad_partials_per_batch(m, nb) * KM_MAX_PARAMS * sizeof(float);
+    // Enough for either form of the first pass (which one runs also depends on the strides).
+    long long rows = param_grad_partials_per_batch(m, nb);
+    const long long feature_rows = param_grad_feature_partials_per_batch(kernel_type, m, nb, c);
+    if (feature_rows > rows) rows = feature_rows;
+    return (size_t)nb * (size_t)rows * KM_MAX_PARAMS * sizeof(float);
 }
 
 // Device scratch of the allocation-free entry point: one array per GPU, held until the

@@ -60,6 +60,72 @@ __device__ __forceinline__ float phase_rev(float f, float x, float c) {
     return __builtin_fmaf(f, lo, __builtin_fmaf(f, hi, -turns));
 }
 
+// Separable form of the Gaussian factor (table kernels): K / sigma is evaluated times
+// 2^KM_TABLE_KSCALE_LOG2, and a chunk of columns may take the form only while every scaled
+// distance of a column to its reference point stays within KM_TABLE_SPAN.
+#define KM_TABLE_KSCALE_LOG2 11
+#define KM_TABLE_SPAN 2.0f
+
+// Separable form of the Gaussian factor: 2^(ra * b + rb) for two neighbouring columns, with
+// ra = 2 a, rb = KS - a^2, a = (x1 - r) s the row's and b = (x2 - r) s the columns' scaled
+// distances to a common reference point r; times the columns' 2^(-b^2) (carried by the rhs
+// operand) this is 2^(KS - ((x1 - x2) s)^2).
+__device__ __forceinline__ void separable_pair_f16(float ra, float rb, float ba, float bb, float one,
+                                                   half2v* hi, half2v* lo) {
+    const float ea = __builtin_amdgcn_exp2f(__builtin_fmaf(ra, ba, rb));
+    const float eb = __builtin_amdgcn_exp2f(__builtin_fmaf(ra, bb, rb));
+    const float2v kv = {ea, eb};
+    const half2v h = __builtin_convertvector(kv, half2v);
+    half2v l;
+    l[0] = (_Float16)__builtin_fmaf(ea, one, -(float)h[0]);
+    l[1] = (_Float16)__builtin_fmaf(eb, one, -(float)h[1]);
+    *hi = h;
+    *lo = l;
+}
+
+__device__ __forceinline__ void split_f16x8(const float (&v)[8], float one, half8v* hi, half8v* lo) {
+    half2v h2[4], l2[4];
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        const float2v p = {v[2 * t], v[2 * t + 1]};
+        h2[t] = __builtin_convertvector(p, half2v);
+        l2[t][0] = (_Float16)__builtin_fmaf(v[2 * t], one, -(float)h2[t][0]);
+        l2[t][1] = (_Float16)__builtin_fmaf(v[2 * t + 1], one, -(float)h2[t][1]);
+    }
+    *hi = join_half2x4(h2);
+    *lo = join_half2x4(l2);
+}
+
+// Minimum and maximum over the wavefront, returned wave-uniform.  Row-wise DPP steps, then the
+// last lane of each row of 16 is carried into the following rows; lane 63 holds the result.
+__device__ __forceinline__ void wave_min_max(float* lo, float* hi) {
+    float a = *lo, b = *hi;
+#define KM_DPP_STEP(ctrl)                                                                              \
+    a = fminf(a, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, a),     \
+                                                                       __builtin_bit_cast(int, a), ctrl, 0xf, 0xf, false))); \
+    b = fmaxf(b, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, b),     \
+                                                                       __builtin_bit_cast(int, b), ctrl, 0xf, 0xf, false)))
+    KM_DPP_STEP(0xb1);   // quad_perm [1, 0, 3, 2]
+    KM_DPP_STEP(0x4e);   // quad_perm [2, 3, 0, 1]
+    KM_DPP_STEP(0x114);  // row_shr 4
+    KM_DPP_STEP(0x118);  // row_shr 8
+    KM_DPP_STEP(0x142);  // row_bcast 15
+    KM_DPP_STEP(0x143);  // row_bcast 31
+#undef KM_DPP_STEP
+    *lo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, a), 63));
+    *hi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, b), 63));
+}
+
+// Largest value over the 4 lanes that share an rhs column (lanes l, l+16, l+32, l+48).
+__device__ __forceinline__ float column_max(float m) {
+    const unsigned bits = __float_as_uint(m);
+    const auto rows = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+    m = fmaxf(__uint_as_float(rows[0]), __uint_as_float(rows[1]));
+    const unsigned bits2 = __float_as_uint(m);
+    const auto halves = __builtin_amdgcn_permlane32_swap(bits2, bits2, false, false);
+    return fmaxf(__uint_as_float(halves[0]), __uint_as_float(halves[1]));
+}
+
 // Per-wavefront view of the problem, shared by the forward kernels.
 struct WaveView {
     long long b;

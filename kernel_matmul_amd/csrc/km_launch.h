@@ -78,6 +78,8 @@ struct ParamGradProblem {
 
 // Partial sums written by the first pass: one row of KM_MAX_PARAMS floats per wavefront.
 long long param_grad_partials_per_batch(int64_t m, long long num_batches);
+// Same for the feature form of the first pass at vector width c (0 where the form does not apply).
+long long param_grad_feature_partials_per_batch(int kernel_type, int64_t m, long long num_batches, int64_t c);
 hipError_t launch_param_grad(const ParamGradProblem& p, hipStream_t stream);
 
 struct IndexProblem {

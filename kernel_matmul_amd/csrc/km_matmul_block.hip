@@ -59,16 +59,6 @@ struct BlockArgs {
     int main_row_blocks;      // row blocks covered by the main items
 };
 
-// Largest value over the 4 lanes that share an rhs column (lanes l, l+16, l+32, l+48).
-__device__ __forceinline__ float column_max(float m) {
-    const unsigned bits = __float_as_uint(m);
-    const auto rows = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
-    m = fmaxf(__uint_as_float(rows[0]), __uint_as_float(rows[1]));
-    const unsigned bits2 = __float_as_uint(m);
-    const auto halves = __builtin_amdgcn_permlane32_swap(bits2, bits2, false, false);
-    return fmaxf(__uint_as_float(halves[0]), __uint_as_float(halves[1]));
-}
-
 __device__ __forceinline__ void read8(const float* p, float (&dst)[8]) {
     const float4v a = *(const float4v*)p;
     const float4v b = *(const float4v*)(p + 4);

@@ -14,6 +14,7 @@
 // (native/common/kernel_function.cuh:221-251).  No atomics: results are reproducible.
 #include "km_batch.h"
 #include "km_common.h"
+#include "km_fwd.h"
 #include "km_launch.h"
 
 namespace km {
@@ -37,44 +38,19 @@ struct GradArgs {
     long long x1_s, x2_s, left_s0, left_s1, right_s0, right_s1, params_s, start_s, end_s;
 };
 
+// One item of the pairwise form: R groups of 16 rows from row0 against the columns
+// [col_begin, col_end), sums written to `prow` (KM_MAX_PARAMS floats).
 // TL > 0: the vector width c is at most 4*TL and the left operand stays in registers.
 // TL == 0: any c; the left operand is re-read (from L1/L2) for every column chunk.
-template <int KT, int TL>
-__global__ void __launch_bounds__(64) param_grad_partial(const GradArgs a) {
-    constexpr int R = 8;
-    const int lane = threadIdx.x;
+template <int KT, int TL, int R>
+__device__ __forceinline__ void pairwise_item(const GradArgs& a, const float* __restrict__ x1,
+                                              const float* __restrict__ x2, const float* __restrict__ left,
+                                              const float* __restrict__ right, const KernelConsts& kc,
+                                              int row0, int col_begin, int col_end,
+                                              float* __restrict__ prow) {
+    const int lane = threadIdx.x & 63;
     const int li = lane & 15;
     const int kk = lane >> 4;
-
-    const long long item = xcd_item(blockIdx.x, a.items_per_xcd);
-    if (item >= a.total_items) {
-        return;
-    }
-    const long long b = item % a.num_batches;
-    const long long rest = item / a.num_batches;
-    const int split = (int)(rest % a.col_splits);
-    const int row_block = (int)(rest / a.col_splits);
-    const int row0 = row_block * KM_BLOCK_SIZE;
-
-    int bidx[KM_MAX_BATCH_RANK];
-    batch_multi_index(a.batch, b, bidx);
-    const float* __restrict__ x1 = a.x1 + batch_offset(a.batch, a.x1_bs, bidx);
-    const float* __restrict__ x2 = a.x2 + batch_offset(a.batch, a.x2_bs, bidx);
-    const float* __restrict__ left = a.left + batch_offset(a.batch, a.left_bs, bidx);
-    const float* __restrict__ right = a.right + batch_offset(a.batch, a.right_bs, bidx);
-    const float* __restrict__ params = a.params + batch_offset(a.batch, a.params_bs, bidx);
-    int range_start = a.start[batch_offset(a.batch, a.start_bs, bidx) + row_block * a.start_s];
-    int range_end = a.end[batch_offset(a.batch, a.end_bs, bidx) + row_block * a.end_s];
-    range_start = max(range_start, 0);
-    range_end = min(range_end, a.n);
-
-    const KernelConsts kc = make_consts<KT>(params, a.params_s, false);
-
-    // Column share of this wavefront, in whole chunks of 16 columns.
-    const int width = max(range_end - range_start, 0);
-    const int per_split = ((width + a.col_splits - 1) / a.col_splits + 15) & ~15;
-    const int col_begin = range_start + split * per_split;
-    const int col_end = min(range_end, col_begin + per_split);
 
     // x1 for the 4 rows per row group this lane owns in the D layout.
     float x1q[R][4];
@@ -156,14 +132,439 @@ __global__ void __launch_bounds__(64) param_grad_partial(const GradArgs a) {
         }
     }
 
-    const long long partial_rows = a.total_items / a.num_batches;
-    float* __restrict__ prow = a.partials + (b * partial_rows + rest) * KM_MAX_PARAMS;
 #pragma unroll
     for (int p = 0; p < KM_MAX_PARAMS; p++) {
         const float total = wave_sum(acc[p]);
         if (lane == 0) {
             prow[p] = total;
         }
+    }
+}
+
+// Per-wavefront decode shared by the two kernels: item -> (batch item, row chunk, column
+// split), the batch item's pointers, and the wavefront's share of the row block's range.
+struct GradItem {
+    long long b, rest;
+    int row0, col_begin, col_end;
+    const float* x1;
+    const float* x2;
+    const float* left;
+    const float* right;
+    const float* params;
+};
+
+__device__ __forceinline__ bool grad_item(const GradArgs& a, int rows_per_item, int col_step, GradItem* g) {
+    const long long item = xcd_item(blockIdx.x, a.items_per_xcd);
+    if (item >= a.total_items) {
+        return false;
+    }
+    g->b = item % a.num_batches;
+    g->rest = item / a.num_batches;
+    const int split = (int)(g->rest % a.col_splits);
+    const int chunk = (int)(g->rest / a.col_splits);
+    const int chunks_per_block = KM_BLOCK_SIZE / rows_per_item;
+    const int row_block = chunk / chunks_per_block;
+    g->row0 = row_block * KM_BLOCK_SIZE + (chunk % chunks_per_block) * rows_per_item;
+
+    int bidx[KM_MAX_BATCH_RANK];
+    batch_multi_index(a.batch, g->b, bidx);
+    g->x1 = a.x1 + batch_offset(a.batch, a.x1_bs, bidx);
+    g->x2 = a.x2 + batch_offset(a.batch, a.x2_bs, bidx);
+    g->left = a.left + batch_offset(a.batch, a.left_bs, bidx);
+    g->right = a.right + batch_offset(a.batch, a.right_bs, bidx);
+    g->params = a.params + batch_offset(a.batch, a.params_bs, bidx);
+    int range_start = a.start[batch_offset(a.batch, a.start_bs, bidx) + row_block * a.start_s];
+    int range_end = a.end[batch_offset(a.batch, a.end_bs, bidx) + row_block * a.end_s];
+    range_start = max(range_start, 0);
+    range_end = min(range_end, a.n);
+    // Column share of this wavefront, in whole steps of col_step columns.
+    const int width = max(range_end - range_start, 0);
+    const int per_split = ((width + a.col_splits - 1) / a.col_splits + col_step - 1) & ~(col_step - 1);
+    g->col_begin = range_start + split * per_split;
+    g->col_end = min(range_end, g->col_begin + per_split);
+    return true;
+}
+
+template <int KT, int TL>
+__global__ void __launch_bounds__(64) param_grad_partial(const GradArgs a) {
+    GradItem g;
+    if (!grad_item(a, KM_BLOCK_SIZE, 16, &g)) {
+        return;
+    }
+    const KernelConsts kc = make_consts<KT>(g.params, a.params_s, false);
+    const long long partial_rows = a.total_items / a.num_batches;
+    pairwise_item<KT, TL, 8>(a, g.x1, g.x2, g.left, g.right, kc, g.row0, g.col_begin, g.col_end,
+                             a.partials + (g.b * partial_rows + g.rest) * KM_MAX_PARAMS);
+}
+
+// ---------------------------------------------------------------------------------------
+// Feature form of pass 1 (rbf and spectral kernels, narrow vector widths).
+//
+// With a reference point c0 per wavefront (the middle row of its rows), h_i = (x1_i - c0) s,
+// g_j = (x2_j - c0) s, A_i / B_j the phases of x1_i - c0 / x2_j - c0 and E_ij the Gaussian
+// factor,  u_ij = h_i - g_j,  cos(A_i - B_j) = cA cB + sA sB,  sin(A_i - B_j) = sA cB - cA sB,
+// every sum the gradient needs is a polynomial in h_i times a row-wise contraction of E with
+// column features F_j = {cB, sB, cB g, sB g, cB g^2, sB g^2} (rbf: {1, g, g^2}):
+//     M[i, c, f] = sum_j E_ij right[j, c] F_jf              T_f[i] = sum_c left[i, c] M[i, c, f]
+//     sum C E cos      = sum_i  cA T0 + sA T1
+//     sum C E cos u^2  = sum_i  cA (h^2 T0 - 2 h T2 + T4) + sA (h^2 T1 - 2 h T3 + T5)
+//     sum C E sin d    = sum_i  [sA (h T0 - T2) - cA (h T1 - T3)] / s
+// M is exactly what the forward table kernel computes for an rhs of (number of features) x c
+// columns: one fma + one exp2 per pair (separable exponent), the hi/lo split, and the
+// split-fp16 MFMAs; the per-pair cosine, sine and the products of the pairwise form are gone.
+// The polynomial in h cancels leading terms of size h^2 against a result of size u^2 ~ 1, so the
+// form is only used while |h_i| <= 12 (measured on 1e5 points: the 22-bit products then leave
+// up to 2e-5 of the gradient's largest component, 1e-6 for |h| <= 6), |g_j| <= 48 (dynamic range
+// of the fp16 operands) and every chunk of columns admits the separable exponent; an item that
+// fails any of these is redone in the pairwise form.
+// ---------------------------------------------------------------------------------------
+#define KM_GF_CHUNK 256
+#define KM_GF_MAX_FEATURES 6
+#define KM_GF_MAX_WIDTH 10 /* widest vector the feature form takes */
+#define KM_GF_TABLE_FLOATS \
+    ((1 + KM_GF_MAX_FEATURES) * KM_GF_CHUNK + KM_GF_CHUNK / 8 + 3 * KM_BLOCK_SIZE + KM_BLOCK_SIZE * KM_GF_MAX_WIDTH)
+#define KM_GF_HMAX 12.0f
+#define KM_GF_GMAX 48.0f
+
+template <int KT, int GE, int R, int TL>
+__global__ void __launch_bounds__(64, 2) param_grad_features(const GradArgs a) {
+    static_assert(KT == KM_KERNEL_RBF || KT == KM_KERNEL_SPECTRAL, "feature form: rbf or spectral");
+    constexpr bool PHASE = KT == KM_KERNEL_SPECTRAL;
+    constexpr int NF = PHASE ? 6 : 3;
+    constexpr int CH = KM_GF_CHUNK;
+    constexpr int KS = KM_TABLE_KSCALE_LOG2;
+    extern __shared__ float lds[];
+    float* tab_b = lds;                    // (x2 - r) s per column, r: reference of its 8 columns
+    float* tab_f = lds + CH;               // [NF][CH] column features times 2^(-b^2)
+    float* tab_ref = lds + (1 + KM_GF_MAX_FEATURES) * CH;
+    float* tab_rows = tab_ref + CH / 8;    // [3][16 R]: cos A, sin A, h per row (epilogue)
+    float* tab_left = tab_rows + 3 * KM_BLOCK_SIZE;  // [16 R][c]: this item's rows of `left` (epilogue)
+
+    GradItem g;
+    if (!grad_item(a, 16 * R, 32, &g)) {
+        return;
+    }
+    const int lane = threadIdx.x;
+    const int li = lane & 15;
+    const int kk = lane >> 4;
+    const KernelConsts kc = make_consts<KT>(g.params, a.params_s, false);
+    const long long partial_rows = a.total_items / a.num_batches;
+    float* __restrict__ prow = a.partials + (g.b * partial_rows + g.rest) * KM_MAX_PARAMS;
+    const int row0 = g.row0;
+    const int col_begin = g.col_begin, col_end = g.col_end;
+
+    // Operand column t = 16 ge + li of group ge holds (feature f, vector column c) = (t / c, t % c).
+    int feat[GE], vcol[GE];
+    bool used[GE];
+    unsigned right_lane[GE];
+#pragma unroll
+    for (int ge = 0; ge < GE; ge++) {
+        const int t = 16 * ge + li;
+        used[ge] = t < NF * a.c;
+        feat[ge] = used[ge] ? t / a.c : 0;
+        vcol[ge] = used[ge] ? t % a.c : 0;
+        right_lane[ge] = (unsigned)(8 * kk * a.right_s0 + vcol[ge] * a.right_s1);
+    }
+
+    float x1v[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        x1v[r] = g.x1[(long long)min(row0 + 16 * r + li, a.m - 1) * a.x1_s];
+    }
+    const float c0 = g.x1[(long long)min(row0 + 8 * R, a.m - 1) * a.x1_s];
+
+    // This item's rows of `left` go to LDS now (coalesced, overlapping the first table) and are
+    // read back in the epilogue; rows past m are zero.
+    for (int e = lane; e < 16 * R * a.c; e += 64) {
+        const int lr = e / a.c, lc = e - lr * a.c;
+        tab_left[e] = row0 + lr < a.m
+                          ? g.left[(long long)(row0 + lr) * a.left_s0 + (long long)lc * a.left_s1]
+                          : 0.0f;
+    }
+
+    float row_lo = __builtin_inff(), row_hi = -__builtin_inff();
+    bool row_nan = false;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        row_lo = fminf(row_lo, x1v[r]);
+        row_hi = fmaxf(row_hi, x1v[r]);
+        row_nan = row_nan || x1v[r] != x1v[r];
+    }
+    wave_min_max(&row_lo, &row_hi);
+    bool ok = !__any(row_nan) && fmaxf(fabsf(row_hi - c0), fabsf(row_lo - c0)) * kc.s <= KM_GF_HMAX;
+
+    int shift[GE];
+    float scale[GE];
+#pragma unroll
+    for (int ge = 0; ge < GE; ge++) {
+        shift[ge] = 100;
+        scale[ge] = used[ge] ? __builtin_ldexpf(1.0f, 100) : 0.0f;
+    }
+    float4v acc[R][GE];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+#pragma unroll
+        for (int ge = 0; ge < GE; ge++) {
+            acc[r][ge] = (float4v){0.0f, 0.0f, 0.0f, 0.0f};
+        }
+    }
+
+    for (int chunk0 = col_begin; ok && chunk0 < col_end; chunk0 += CH) {
+        const int chunk_end = min(chunk0 + CH, col_end);
+        const int padded = (chunk_end - chunk0 + 31) & ~31;
+        const float* x2c = g.x2 + (long long)chunk0 * a.x2_s;
+        const unsigned x2_stride = (unsigned)a.x2_s;
+        const int last = chunk_end - 1 - chunk0;
+        // All loads of the chunk first (4 columns per lane and the reference point of column
+        // group `lane`), staged through the feature area of the table.
+        {
+            float xq[CH / 64];
+#pragma unroll
+            for (int i = 0; i < CH / 64; i++) {
+                xq[i] = x2c[(unsigned long long)(unsigned)min(lane + 64 * i, last) * x2_stride];
+            }
+            const float ref_own = x2c[(unsigned long long)(unsigned)min(8 * (lane & 31) + 4, last) * x2_stride];
+#pragma unroll
+            for (int i = 0; i < CH / 64; i++) {
+                tab_b[lane + 64 * i] = xq[i];
+            }
+            if (lane < CH / 8) {
+                tab_ref[lane] = ref_own;
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+        bool cols_ok = true;
+        float lo = row_lo, hi = row_hi;
+#pragma unroll 1
+        for (int q = lane; q < padded; q += 64) {
+            const float xv = tab_b[q];
+            const float ref = tab_ref[q >> 3];
+            const float xd = xv - ref;
+            const float bb = xd - xv;
+            const float err = (xv - (xd - bb)) - (ref + bb);  // exact rounding error of xd
+            const float b = xd * kc.s;
+            const float gq = (xv - c0) * kc.s;
+            const float wgt = __builtin_amdgcn_exp2f(-b * b);
+            float p0 = wgt, p1 = 0.0f;
+            if (PHASE) {
+                const float th = phase_rev(kc.f, xv, c0);
+                p0 = wgt * __builtin_amdgcn_cosf(th);
+                p1 = wgt * __builtin_amdgcn_sinf(th);
+            }
+            tab_b[q] = b;
+            if (PHASE) {
+                tab_f[0 * CH + q] = p0;
+                tab_f[1 * CH + q] = p1;
+                tab_f[2 * CH + q] = p0 * gq;
+                tab_f[3 * CH + q] = p1 * gq;
+                tab_f[4 * CH + q] = p0 * gq * gq;
+                tab_f[5 * CH + q] = p1 * gq * gq;
+            } else {
+                tab_f[0 * CH + q] = p0;
+                tab_f[1 * CH + q] = p0 * gq;
+                tab_f[2 * CH + q] = p0 * gq * gq;
+            }
+            cols_ok = cols_ok && err == 0.0f && fabsf(b) <= KM_TABLE_SPAN && fabsf(gq) <= KM_GF_GMAX;
+            lo = fminf(lo, ref);
+            hi = fmaxf(hi, ref);
+        }
+        wave_min_max(&lo, &hi);
+        // x1 - r is exact for every row and reference point when all coordinates involved have
+        // one sign and their spread does not exceed the smallest magnitude.
+        const bool rows_ok = (lo > 0.0f || hi < 0.0f) && (hi - lo) <= fminf(fabsf(lo), fabsf(hi));
+        ok = __all(cols_ok) && rows_ok;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        if (!ok) {
+            break;
+        }
+
+        // Steps of 32 columns.  The operands of a step are requested at its start (no prefetch:
+        // the registers go to the accumulators; other wavefronts cover the latency).
+        float raw[GE][8];
+        auto load = [&](int c0s) {
+            if (c0s + 32 <= chunk_end) {
+                const float* ru = g.right + (long long)c0s * a.right_s0;
+#pragma unroll
+                for (int t = 0; t < 8; t++) {
+#pragma unroll
+                    for (int ge = 0; ge < GE; ge++) {
+                        raw[ge][t] = (ru + t * a.right_s0)[right_lane[ge]];
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int t = 0; t < 8; t++) {
+                    const int col = c0s + 8 * kk + t;
+                    const int colc = min(col, chunk_end - 1);
+#pragma unroll
+                    for (int ge = 0; ge < GE; ge++) {
+                        const float v = g.right[(long long)colc * a.right_s0 + vcol[ge] * a.right_s1];
+                        raw[ge][t] = col < chunk_end ? v : 0.0f;
+                    }
+                }
+            }
+        };
+        load(chunk0);
+        for (int c0s = chunk0; c0s < chunk_end; c0s += 32) {
+            const int off = c0s - chunk0 + 8 * kk;
+            float bv[8];
+            {
+                const float4v v0 = *(const float4v*)(tab_b + off);
+                const float4v v1 = *(const float4v*)(tab_b + off + 4);
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    bv[u] = v0[u];
+                    bv[4 + u] = v1[u];
+                }
+            }
+            const float ref = tab_ref[off >> 3];
+            half8v bhi[GE], blo[GE];
+#pragma unroll
+            for (int ge = 0; ge < GE; ge++) {
+                const float* fp = tab_f + feat[ge] * CH + off;
+                const float4v m0 = *(const float4v*)fp;
+                const float4v m1 = *(const float4v*)(fp + 4);
+                // Largest magnitude of this operand column over the step (the 4 lanes that share
+                // it hold 8 columns each), features included (they are not bounded by one).
+                float rv[8];
+                float m = 0.0f;
+#pragma unroll
+                for (int t = 0; t < 8; t++) {
+                    rv[t] = raw[ge][t] * (t < 4 ? m0[t & 3] : m1[t & 3]);
+                    m = fmaxf(m, fabsf(rv[t]));
+                }
+                m = column_max(m);
+                const bool grow = used[ge] && !(m * scale[ge] < 32768.0f);
+                if (__any(grow)) {
+                    if (grow) {
+                        // m < 2^e, so m * 2^(14 - e) < 2^14.
+                        const int e = __builtin_amdgcn_frexp_expf(m);
+                        const int new_shift = min(max(14 - e, -100), 100);
+                        const float factor = __builtin_ldexpf(1.0f, new_shift - shift[ge]);
+#pragma unroll
+                        for (int r = 0; r < R; r++) {
+                            acc[r][ge] *= factor;
+                        }
+                        shift[ge] = new_shift;
+                        scale[ge] = __builtin_ldexpf(1.0f, new_shift);
+                    }
+                }
+#pragma unroll
+                for (int t = 0; t < 8; t++) {
+                    rv[t] *= scale[ge];
+                }
+                split_f16x8(rv, kc.one, &bhi[ge], &blo[ge]);
+            }
+            if (c0s + 32 < chunk_end) {
+                load(c0s + 32);
+            }
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                half2v h2[4], l2[4];
+                const float av = (x1v[r] - ref) * kc.s;
+                const float ra = av + av;
+                const float rb = __builtin_fmaf(-av, av, (float)KS);
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    separable_pair_f16(ra, rb, bv[2 * t], bv[2 * t + 1], kc.one, &h2[t], &l2[t]);
+                }
+                const half8v ahi = join_half2x4(h2);
+                const half8v alo = join_half2x4(l2);
+#pragma unroll
+                for (int ge = 0; ge < GE; ge++) {
+                    acc[r][ge] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahi, bhi[ge], acc[r][ge], 0, 0, 0);
+                    acc[r][ge] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahi, blo[ge], acc[r][ge], 0, 0, 0);
+                    acc[r][ge] = __builtin_amdgcn_mfma_f32_16x16x32_f16(alo, bhi[ge], acc[r][ge], 0, 0, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        // All reads of the table are done before the next chunk overwrites it.
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    }
+
+    if (!ok) {
+        // Outside the conditions of the feature form: this item in the pairwise form.
+        pairwise_item<KT, TL, R>(a, g.x1, g.x2, g.left, g.right, kc, row0, col_begin, col_end, prow);
+        return;
+    }
+
+    // Rows: cos A, sin A and h, by the lanes that hold the coordinates (A layout), read back in
+    // the D layout (rows 16 r + 4 kk + v).
+    if (kk == 0) {
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            float ca = 1.0f, sa = 0.0f;
+            if (PHASE) {
+                const float th = phase_rev(kc.f, x1v[r], c0);
+                ca = __builtin_amdgcn_cosf(th);
+                sa = __builtin_amdgcn_sinf(th);
+            }
+            tab_rows[16 * r + li] = ca;
+            tab_rows[16 * R + 16 * r + li] = sa;
+            tab_rows[32 * R + 16 * r + li] = (x1v[r] - c0) * kc.s;
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f;
+    int pw[GE];        // power of g in the lane's feature of group ge
+    bool odd[GE];      // sin B (odd) or cos B (even) feature
+    float unscale[GE];
+#pragma unroll
+    for (int ge = 0; ge < GE; ge++) {
+        pw[ge] = PHASE ? (feat[ge] >> 1) : feat[ge];
+        odd[ge] = PHASE && (feat[ge] & 1);
+        unscale[ge] = used[ge] ? __builtin_ldexpf(1.0f, -shift[ge] - KS) : 0.0f;
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const float4v ca4 = *(const float4v*)(tab_rows + 16 * r + 4 * kk);
+        const float4v sa4 = *(const float4v*)(tab_rows + 16 * R + 16 * r + 4 * kk);
+        const float4v h4 = *(const float4v*)(tab_rows + 32 * R + 16 * r + 4 * kk);
+#pragma unroll
+        for (int ge = 0; ge < GE; ge++) {
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const float lv = tab_left[(16 * r + 4 * kk + v) * a.c + vcol[ge]];
+                const float val = acc[r][ge][v] * unscale[ge] * lv;
+                const float h = h4[v];
+                const float poly = pw[ge] == 0 ? h * h : (pw[ge] == 1 ? -2.0f * h : 1.0f);  // of (h - g)^2
+                if (PHASE) {
+                    const float base = odd[ge] ? sa4[v] : ca4[v];   // cos(A - B): cA cB + sA sB
+                    const float alt = odd[ge] ? -ca4[v] : sa4[v];   // sin(A - B): sA cB - cA sB
+                    const float lin = pw[ge] == 0 ? h : (pw[ge] == 1 ? -1.0f : 0.0f);  // of (h - g)
+                    s0 = __builtin_fmaf(base * poly, val, s0);
+                    s1 = __builtin_fmaf(alt * lin, val, s1);
+                    s2 = __builtin_fmaf(pw[ge] == 0 ? base : 0.0f, val, s2);
+                } else {
+                    s0 = __builtin_fmaf(poly, val, s0);
+                    s1 = __builtin_fmaf(pw[ge] == 0 ? 1.0f : 0.0f, val, s1);
+                }
+            }
+        }
+        // One row group at a time (registers).
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    if (PHASE) {
+        s1 *= fabsf(g.params[0]) * (1.0f / KM_SQRT_HALF_LOG2E);  // d = u / s
+    }
+    s0 = wave_sum(s0);
+    s1 = wave_sum(s1);
+    s2 = wave_sum(s2);
+    if (lane == 0) {
+        prow[0] = s0;
+        prow[1] = s1;
+        prow[2] = PHASE ? s2 : 0.0f;
+        prow[3] = 0.0f;
     }
 }
 
@@ -219,11 +620,9 @@ __global__ void __launch_bounds__(256) param_grad_reduce(const ReduceArgs a) {
 // ---------------------------------------------------------------------------------------
 // Host dispatch.
 // ---------------------------------------------------------------------------------------
-static int grad_col_splits(int64_t m, long long num_batches) {
+static int grad_col_splits(long long base) {
     // Enough wavefronts to populate the 1024 SIMDs of the device several times over when the
-    // row-block count alone does not.
-    const long long row_blocks = (m + KM_BLOCK_SIZE - 1) / KM_BLOCK_SIZE;
-    const long long base = row_blocks * num_batches;
+    // row-chunk count alone does not.
     if (base <= 0) {
         return 1;
     }
@@ -235,7 +634,59 @@ static int grad_col_splits(int64_t m, long long num_batches) {
 
 long long param_grad_partials_per_batch(int64_t m, long long num_batches) {
     const long long row_blocks = (m + KM_BLOCK_SIZE - 1) / KM_BLOCK_SIZE;
-    return row_blocks * grad_col_splits(m, num_batches);
+    return row_blocks * grad_col_splits(row_blocks * num_batches);
+}
+
+// Decomposition of the feature form for a vector width c, or GE = 0 when the form does not
+// apply (locally periodic kernel, wide vectors).  GE groups of 16 operand columns hold the
+// (number of features) x c products; wide operands get fewer rows per wavefront.
+struct FeaturePlan {
+    int GE, R, TL;
+};
+
+static FeaturePlan feature_plan(int kernel_type, int64_t c) {
+    FeaturePlan f = {0, 8, 0};
+    const int features = kernel_type == KM_KERNEL_SPECTRAL ? 6 : (kernel_type == KM_KERNEL_RBF ? 3 : 0);
+    // Up to 32 operand columns: with more, the accumulators leave room for 64 rows per wavefront
+    // only, and measured (spectral, c = 8) that is slower than the pairwise form.
+    if (features == 0 || c <= 0 || features * c > 32) {
+        return f;
+    }
+    f.GE = (int)((features * c + 15) / 16);
+    f.R = 8;
+    f.TL = c <= 4 ? 1 : (c <= 8 ? 2 : 4);
+    return f;
+}
+
+long long param_grad_feature_partials_per_batch(int kernel_type, int64_t m, long long num_batches, int64_t c) {
+    const FeaturePlan f = feature_plan(kernel_type, c);
+    if (f.GE == 0) {
+        return 0;
+    }
+    const long long row_blocks = (m + KM_BLOCK_SIZE - 1) / KM_BLOCK_SIZE;
+    const long long chunks = row_blocks * (8 / f.R);
+    return chunks * grad_col_splits(chunks * num_batches);
+}
+
+template <int KT, int GE, int R, int TL>
+static hipError_t launch_features_as(const GradArgs& a, unsigned grid_x, hipStream_t stream) {
+    hipLaunchKernelGGL((param_grad_features<KT, GE, R, TL>), dim3(grid_x), dim3(64),
+                       KM_GF_TABLE_FLOATS * sizeof(float), stream, a);
+    return hipGetLastError();
+}
+
+static hipError_t launch_features(int kernel_type, const FeaturePlan& f, const GradArgs& a, unsigned grid_x,
+                                  hipStream_t stream) {
+    if (kernel_type == KM_KERNEL_SPECTRAL) {  // 6 features: c <= 5
+        if (f.GE == 1) return launch_features_as<KM_KERNEL_SPECTRAL, 1, 8, 1>(a, grid_x, stream);
+        if (f.TL == 1) return launch_features_as<KM_KERNEL_SPECTRAL, 2, 8, 1>(a, grid_x, stream);
+        return launch_features_as<KM_KERNEL_SPECTRAL, 2, 8, 2>(a, grid_x, stream);
+    }
+    // rbf, 3 features: c <= 10
+    if (f.GE == 1 && f.TL == 1) return launch_features_as<KM_KERNEL_RBF, 1, 8, 1>(a, grid_x, stream);
+    if (f.GE == 1) return launch_features_as<KM_KERNEL_RBF, 1, 8, 2>(a, grid_x, stream);
+    if (f.TL == 2) return launch_features_as<KM_KERNEL_RBF, 2, 8, 2>(a, grid_x, stream);
+    return launch_features_as<KM_KERNEL_RBF, 2, 8, 4>(a, grid_x, stream);
 }
 
 template <int KT>
@@ -291,9 +742,23 @@ hipError_t launch_param_grad(const ParamGradProblem& p, hipStream_t stream) {
     a.m = (int)p.m;
     a.n = (int)p.n;
     a.c = (int)p.c;
-    a.col_splits = grad_col_splits(p.m, p.num_batches);
     const long long row_blocks = (p.m + KM_BLOCK_SIZE - 1) / KM_BLOCK_SIZE;
-    a.total_items = row_blocks * a.col_splits * p.num_batches;
+    // Feature form where it applies (its 32-bit lane offsets need moderate, non-negative strides
+    // of `right`); pairwise form otherwise.
+    FeaturePlan fplan = feature_plan(p.kernel_type, p.c);
+    {
+        const int64_t r0 = p.right_strides[r], r1 = p.right_strides[r + 1];
+        if (r0 < 0 || r1 < 0 || r0 > (1 << 24) || r1 > (1 << 24) || p.x2_strides[r] < 0 ||
+            p.x2_strides[r] > (1 << 24)) {
+            fplan.GE = 0;
+        }
+    }
+    long long chunks = row_blocks;
+    if (fplan.GE > 0) {
+        chunks = row_blocks * (8 / fplan.R);
+    }
+    a.col_splits = grad_col_splits(chunks * p.num_batches);
+    a.total_items = chunks * a.col_splits * p.num_batches;
     a.items_per_xcd = (a.total_items + KM_NUM_XCD - 1) / KM_NUM_XCD;
     a.x1 = p.x1;
     a.x2 = p.x2;
@@ -314,7 +779,12 @@ hipError_t launch_param_grad(const ParamGradProblem& p, hipStream_t stream) {
     a.end_s = p.end_strides[r];
 
     const unsigned grid_x = (unsigned)(a.items_per_xcd * KM_NUM_XCD);
-    if (grid_x > 0) {  // no rows: the reduce pass alone writes the zero gradient
+    if (grid_x > 0 && fplan.GE > 0) {
+        const hipError_t err = launch_features(p.kernel_type, fplan, a, grid_x, stream);
+        if (err != hipSuccess) {
+            return err;
+        }
+    } else if (grid_x > 0) {  // no rows: the reduce pass alone writes the zero gradient
         hipError_t err;
         switch (p.kernel_type) {
             case KM_KERNEL_RBF: err = launch_partial<KM_KERNEL_RBF>(a, grid_x, stream); break;
@@ -326,7 +796,7 @@ hipError_t launch_param_grad(const ParamGradProblem& p, hipStream_t stream) {
         }
     }
 
-    return launch_param_grad_reduce(p.kernel_type, a.batch, p.num_batches, row_blocks * a.col_splits,
+    return launch_param_grad_reduce(p.kernel_type, a.batch, p.num_batches, chunks * a.col_splits,
                                     a.partials, p.params, a.params_bs, a.params_s, p.grad, stream);
 }
 

@@ -535,3 +535,53 @@ def test_entry_operators_phase_beyond_256_revolutions(kernel_type):
     gtol = _grad_tolerance(gexp) + 4 * phase_eps * bound
     assert np.all(gerr <= gtol), (ggot.cpu().numpy(), gexp, gerr / gtol)
     del one
+
+
+# The parameter gradient takes a feature form (moments of the columns about a reference point
+# per wavefront) only where that loses nothing and redoes the other row blocks pair by pair:
+# exact coordinate differences, rows within 12 and columns within 48 scaled lengths of the
+# reference point.  Every regime must meet the tolerance, whichever form its row blocks take.
+GRADIENT_REGIMES = dict(COORDINATE_REGIMES)
+GRADIENT_REGIMES.update({
+    "sparse_rows": (50.0, 6000.0, True),     # a row block spans hundreds of lengthscales
+    "dense_rows": (50.0, 15.0, True),        # everything within a few lengthscales
+})
+
+
+@pytest.mark.parametrize("vector_width", [3, 5, 8])
+@pytest.mark.parametrize("kernel_type", ["rbf", "spectral", "locally_periodic"])
+@pytest.mark.parametrize("regime", sorted(GRADIENT_REGIMES))
+def test_param_grad_coordinate_regimes(regime, kernel_type, vector_width):
+    from kernel_matmul_amd.ranges import make_ranges
+    from tests.conftest import make_params
+
+    offset, extent, is_sorted = GRADIENT_REGIMES[regime]
+    g = torch.Generator().manual_seed(12)
+    m, batch = 1500, (2,)
+    x = torch.rand(m, generator=g) * extent + offset
+    if is_sorted:
+        x = torch.sort(x)[0]
+        if regime == "from_zero":
+            x[0] = 0.0
+        x1 = x2 = x
+        start, end = make_ranges(2.5 if extent < 1000 else 12.0, x)
+    else:
+        x1 = torch.sort(x)[0]
+        x2 = x[torch.randperm(m, generator=g)]
+        rows = (m + 127) // 128
+        start = torch.zeros(rows, dtype=torch.int32)
+        end = torch.full((rows,), m, dtype=torch.int32)
+    left = torch.randn(*batch, m, vector_width, generator=g)
+    left = left / torch.linalg.norm(left, dim=-2, keepdim=True)
+    right = torch.randn(m, vector_width, generator=g)
+    right = right / torch.linalg.norm(right, dim=-2, keepdim=True)
+    params = make_params(kernel_type, batch)
+    device = torch.device("cuda:0")
+    expand = lambda t: t.to(device).expand(*batch, *t.shape)
+    args = (expand(x1), expand(x2), left.to(device), expand(right), params.to(device), expand(start), expand(end))
+    result = load_native("bilinear_derivative",
+                         BilinearDerivativeConfiguration(kernel_type).make_config(args)).call(*args)
+    f = lambda t: t.detach().cpu().numpy()
+    expected = oracle.param_grad(kernel_type, *(f(t) for t in args))
+    err = np.abs(result.cpu().double().numpy() - expected)
+    assert np.all(err <= _grad_tolerance(expected)), (result.cpu().numpy(), expected)
