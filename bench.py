@@ -49,8 +49,8 @@ WORKLOADS = {
 
 # HBM bytes per launch of the headline kernel, from the FETCH_SIZE / WRITE_SIZE counter runs
 # summarised in the file named here (an offline rocprofv3 --pmc run, not measured by this script).
-TRAFFIC_SOURCE = "profiles/fwd_table_f16_headline_counters.md"
-MEASURED_TRAFFIC_BYTES = {"headline": 58763674}
+TRAFFIC_SOURCE = "profiles/fwd_table_f16_grouped_headline_counters.md"
+MEASURED_TRAFFIC_BYTES = {"headline": 58506240}
 
 FLOPS_PER_PAIR = {"rbf": lambda k: 5 + 2 * k, "spectral": lambda k: 8 + 2 * k,
                   "locally_periodic": lambda k: 10 + 2 * k}

@@ -67,9 +67,9 @@ __device__ __forceinline__ float phase_rev(float f, float x, float c) {
 #define KM_TABLE_SPAN 2.0f
 
 // Separable form of the Gaussian factor: 2^(ra * b + rb) for two neighbouring columns, with
-// ra = 2 a, rb = KS - a^2, a = (x1 - r) s the row's and b = (x2 - r) s the columns' scaled
-// distances to a common reference point r; times the columns' 2^(-b^2) (carried by the rhs
-// operand) this is 2^(KS - ((x1 - x2) s)^2).
+// ra * b = 2 a b (the factor 2 carried by either operand), rb = KS - a^2, a = (x1 - r) s the
+// row's and b = (x2 - r) s the columns' scaled distances to a common reference point r; times
+// the columns' 2^(-b^2) (carried by the rhs operand) this is 2^(KS - ((x1 - x2) s)^2).
 __device__ __forceinline__ void separable_pair_f16(float ra, float rb, float ba, float bb, float one,
                                                    half2v* hi, half2v* lo) {
     const float ea = __builtin_amdgcn_exp2f(__builtin_fmaf(ra, ba, rb));

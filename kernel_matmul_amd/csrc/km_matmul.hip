@@ -402,11 +402,10 @@ __device__ __forceinline__ void f16_step(const float (&x2v)[8], const float (&ra
         if (SEP) {
             // Row constants for this lane's 8 columns (ref: their reference point).
             const float av = (x1v[r] - ref) * kc.s;
-            const float ra = av + av;
             const float rb = __builtin_fmaf(-av, av, (float)KS);
 #pragma unroll
             for (int t = 0; t < 4; t++) {
-                separable_pair_f16(ra, rb, x2v[2 * t], x2v[2 * t + 1], kc.one, &h2[t], &l2[t]);
+                separable_pair_f16(av, rb, x2v[2 * t], x2v[2 * t + 1], kc.one, &h2[t], &l2[t]);
             }
         } else {
 #pragma unroll
@@ -754,11 +753,13 @@ __device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds,
         const bool rows_ok = rows_finite && (lo > 0.0f || hi < 0.0f) && (hi - lo) <= fminf(fabsf(lo), fabsf(hi));
         const bool separable = allow && __all(cols_ok) && rows_ok;
         if (separable) {
-            // The column factor 2^(-b^2) of the separable form joins the phase factors.
+            // The column factor 2^(-b^2) of the separable form joins the phase factors, and the
+            // table keeps 2 b, the form the rows' exponent takes it in.
 #pragma unroll 1
             for (int q = lane; q < padded; q += 64) {
                 const float b = tab_b[q];
                 const float wgt = __builtin_amdgcn_exp2f(-b * b);
+                tab_b[q] = b + b;
                 tab_cos[q] *= wgt;
                 if (PHASE) {
                     tab_sin[q] *= wgt;
