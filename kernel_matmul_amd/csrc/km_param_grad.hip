@@ -3,8 +3,12 @@
 // native/matmul_bwd/matmul_bwd.cu:12-221) and bilinear_derivative
 // (native/bilinear_derivative/bilinear_derivative.cu:12-183), which compute the same sum.
 //
-// Pass 1 (param_grad_partial): a wavefront owns 128 rows and a share of the row block's
-// column range.  Per 16-column chunk and 16-row group the coefficient tile C (16x16) is
+// Pass 1 has two forms.  Feature form (param_grad_features, rbf and spectral kernels with
+// narrow vectors; described at the kernel): the sums are polynomials in the rows' coordinate
+// times contractions of the Gaussian factor with a handful of column features, computed like
+// the forward table kernel.  Pairwise form (param_grad_partial, every kernel; also the
+// per-item fallback of the feature form): a wavefront owns 128 rows and a share of the row
+// block's column range.  Per 16-column chunk and 16-row group the coefficient tile C (16x16) is
 // formed on the matrix pipe from left/right (v_mfma_f32_16x16x4_f32 over the vector
 // columns); its D layout gives each lane 4 (row, col) pairs, for which the lane evaluates
 // the kernel derivatives and accumulates per-lane sums.  The sums are combined across the
