@@ -22,6 +22,10 @@ def _flatten(t: Tensor) -> Tensor:
     return t.reshape(-1, t.shape[-1])
 
 
+def _ascending(t: Tensor) -> bool:
+    return t.shape[-1] < 2 or bool(torch.all(t[..., 1:] >= t[..., :-1]))
+
+
 def make_ranges(
     cutoff: float | None,
     x1: Tensor,
@@ -29,8 +33,14 @@ def make_ranges(
     *,
     block_size: int = _BLOCK_SIZE,
     align: bool = False,
+    check_sorted: bool = False,
 ) -> tuple[Tensor, Tensor]:
     """Compute the sparsity pattern for a cutoff distance.
+
+    Inputs are expected sorted ascending along their last dimension.  Host tensors go through
+    the sequential scan of the reference (native/ranges/ranges.cpp:8-101), which returns some
+    pattern for unsorted data too; GPU tensors are processed on the GPU by binary searches
+    that agree with the scan bit for bit on sorted data only.
 
     Args:
         cutoff: entries with ``|x1[i] - x2[j]| > cutoff`` may be dropped; ``None`` keeps all.
@@ -40,6 +50,8 @@ def make_ranges(
         block_size: rows per block.
         align: restrict start/end to multiples of ``block_size`` (or ``n2``) so that the
             pattern can be transposed exactly.
+        check_sorted: verify GPU inputs (one host synchronisation) and run unsorted ones
+            through the host scan, so that the result never depends on the tensors' device.
 
     Returns:
         ``(start, end)``, int32 tensors of shape ``(batch..., ceil(n1 / block_size))`` on
@@ -55,7 +67,14 @@ def make_ranges(
         start = torch.zeros(x1f.shape[0], rows, dtype=torch.int32, device=x1.device)
         end = torch.full((x1f.shape[0], rows), n2, dtype=torch.int32, device=x1.device)
     else:
-        start, end = _native.make_ranges_2d(x1f, x2f, cutoff, block_size, align)
+        if check_sorted and x1f.is_cuda and not (_ascending(x1f) and (x2f is None or _ascending(x2f))):
+            device = x1f.device
+            start, end = _native.make_ranges_2d(
+                x1f.cpu(), x2f.cpu() if x2f is not None else None, cutoff, block_size, align
+            )
+            start, end = start.to(device), end.to(device)
+        else:
+            start, end = _native.make_ranges_2d(x1f, x2f, cutoff, block_size, align)
 
     return start.reshape(*batch_shape, rows), end.reshape(*batch_shape, rows)
 
