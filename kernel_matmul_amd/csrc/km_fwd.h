@@ -60,6 +60,17 @@ __device__ __forceinline__ float phase_rev(float f, float x, float c) {
     return __builtin_fmaf(f, lo, __builtin_fmaf(f, hi, -turns));
 }
 
+// fp16 roundings of the residuals a0 * b0 - h[0], a1 * b1 - h[1] of two products against their
+// fp16 values h (the low halves of the hi + lo split).  Written as two fp32 results (one
+// v_fma_mix_f32 each, reading the fp16 operand directly) rounded together by one
+// v_cvt_pk_f16_f32: measured on gfx950, v_fma_mixlo_f16 / v_fma_mixhi_f16, which would round
+// inside the fused instruction, issue at half the rate of v_fma_mix_f32, so the two-instruction
+// form per value pair costs a fifth more than these three.
+__device__ __forceinline__ half2v residual_f16x2(float a0, float b0, float a1, float b1, half2v h) {
+    const float2v res = {__builtin_fmaf(a0, b0, -(float)h[0]), __builtin_fmaf(a1, b1, -(float)h[1])};
+    return __builtin_convertvector(res, half2v);
+}
+
 // Separable form of the Gaussian factor (table kernels): K / sigma is evaluated times
 // 2^KM_TABLE_KSCALE_LOG2, and a chunk of columns may take the form only while every scaled
 // distance of a column to its reference point stays within KM_TABLE_SPAN.
@@ -76,11 +87,8 @@ __device__ __forceinline__ void separable_pair_f16(float ra, float rb, float ba,
     const float eb = __builtin_amdgcn_exp2f(__builtin_fmaf(ra, bb, rb));
     const float2v kv = {ea, eb};
     const half2v h = __builtin_convertvector(kv, half2v);
-    half2v l;
-    l[0] = (_Float16)__builtin_fmaf(ea, one, -(float)h[0]);
-    l[1] = (_Float16)__builtin_fmaf(eb, one, -(float)h[1]);
     *hi = h;
-    *lo = l;
+    *lo = residual_f16x2(ea, one, eb, one, h);
 }
 
 __device__ __forceinline__ void split_f16x8(const float (&v)[8], float one, half8v* hi, half8v* lo) {
@@ -89,8 +97,7 @@ __device__ __forceinline__ void split_f16x8(const float (&v)[8], float one, half
     for (int t = 0; t < 4; t++) {
         const float2v p = {v[2 * t], v[2 * t + 1]};
         h2[t] = __builtin_convertvector(p, half2v);
-        l2[t][0] = (_Float16)__builtin_fmaf(v[2 * t], one, -(float)h2[t][0]);
-        l2[t][1] = (_Float16)__builtin_fmaf(v[2 * t + 1], one, -(float)h2[t][1]);
+        l2[t] = residual_f16x2(v[2 * t], one, v[2 * t + 1], one, h2[t]);
     }
     *hi = join_half2x4(h2);
     *lo = join_half2x4(l2);

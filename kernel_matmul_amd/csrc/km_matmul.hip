@@ -281,16 +281,11 @@ __device__ __forceinline__ void kernel_pair_f16(float x1, float x2a, float x2b, 
         kv[t] = KT == KM_KERNEL_SPECTRAL ? ea[t] * ca[t] : ea[t];
     }
     const half2v h = __builtin_convertvector(kv, half2v);
-    half2v l;
-#pragma unroll
-    for (int t = 0; t < 2; t++) {
-        // Residual of the exact product where there is one, computed and rounded to fp16 by
-        // one v_fma_mixlo/hi_f16 (the fp16 operand is read directly).  `one` is a run-time
-        // 1.0 that keeps the expression an fma.
-        l[t] = (_Float16)__builtin_fmaf(ea[t], KT == KM_KERNEL_SPECTRAL ? ca[t] : one, -(float)h[t]);
-    }
+    // Residuals of the exact products where there is one (`one` is a run-time 1.0 that keeps
+    // the expression a fused multiply-add reading the fp16 operand directly).
     *hi = h;
-    *lo = l;
+    *lo = residual_f16x2(ea[0], KT == KM_KERNEL_SPECTRAL ? ca[0] : one, ea[1],
+                         KT == KM_KERNEL_SPECTRAL ? ca[1] : one, h);
 }
 
 // Operands of one step of 32 columns for this lane: x2 and rhs at columns c0 + 8 kk + t.

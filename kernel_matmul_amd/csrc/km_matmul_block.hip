@@ -75,8 +75,7 @@ __device__ __forceinline__ void split8(const float (&v)[8], float one, half8v* h
     for (int t = 0; t < 4; t++) {
         const float2v p = {v[2 * t], v[2 * t + 1]};
         h2[t] = __builtin_convertvector(p, half2v);
-        l2[t][0] = (_Float16)__builtin_fmaf(v[2 * t], one, -(float)h2[t][0]);
-        l2[t][1] = (_Float16)__builtin_fmaf(v[2 * t + 1], one, -(float)h2[t][1]);
+        l2[t] = residual_f16x2(v[2 * t], one, v[2 * t + 1], one, h2[t]);
     }
     *hi = join_half2x4(h2);
     *lo = join_half2x4(l2);
@@ -127,11 +126,8 @@ __device__ __forceinline__ void block_eval(const float (&xa)[2], const float (&p
             }
             const float2v kv = {COS ? ea[0] * ca[0] : ea[0], COS ? ea[1] * ca[1] : ea[1]};
             h2[t2] = __builtin_convertvector(kv, half2v);
-#pragma unroll
-            for (int h = 0; h < 2; h++) {
-                // Residual of the exact product, one fused instruction reading the fp16 half.
-                l2[t2][h] = (_Float16)__builtin_fmaf(ea[h], COS ? ca[h] : kc.one, -(float)h2[t2][h]);
-            }
+            // Residuals of the exact products (fused, reading the fp16 halves directly).
+            l2[t2] = residual_f16x2(ea[0], COS ? ca[0] : kc.one, ea[1], COS ? ca[1] : kc.one, h2[t2]);
         }
         const half8v ahi = join_half2x4(h2);
         const half8v alo = join_half2x4(l2);
