@@ -93,7 +93,7 @@ class Prepared:
     """One workload resident on the GPU, ready to be called."""
 
     def __init__(self, name, device, batch_override=None, variant="auto", rows_per_wave=0, col_splits=0,
-                 tail_balance=True, group_tail=None):
+                 tail_balance=True, group_tail=None, group_tail_halves=None):
         import torch
 
         from kernel_matmul_amd.compile import load_native
@@ -138,6 +138,8 @@ class Prepared:
             defines["MATMUL_TAIL_BALANCE"] = 0
         if group_tail is not None:
             defines["MATMUL_GROUP_TAIL"] = group_tail
+            if group_tail_halves is not None:
+                defines["MATMUL_GROUP_TAIL_HALVES"] = group_tail_halves
         self.op = load_native("matmul", defines)
         self.kernel = self.op.describe(*self.args)
         if self.is_grad:
@@ -255,6 +257,8 @@ def main() -> int:
     ap.add_argument("--no-tail-balance", action="store_true")
     ap.add_argument("--group-tail", type=int, default=None,
                     help="table kernel: grouped launch with this many column-split items per XCD")
+    ap.add_argument("--group-tail-halves", type=int, default=None,
+                    help="with --group-tail: how many of those items also run as two halves of 64 rows")
     ap.add_argument("--no-cpu-baseline", action="store_true",
                     help="skip the host-side legs: the CPU baseline and the float64 error figures")
     ap.add_argument("--no-configs", action="store_true", help="skip the other benchmark configurations")
@@ -280,7 +284,7 @@ def main() -> int:
     device = torch.device("cuda:0")
 
     main_run = Prepared(args.workload, device, args.batch, args.variant, args.rows_per_wave, args.col_splits,
-                        not args.no_tail_balance, args.group_tail)
+                        not args.no_tail_balance, args.group_tail, args.group_tail_halves)
     w = main_run.w
     n, batch = w["n"], w["batch"]
 

@@ -64,9 +64,10 @@ typedef struct km_launch_options {
     int rows_per_wave;    /* 0 = table; else 16, 32, 64 or 128 rows of x1 per wavefront */
     int col_splits;       /* 0 = table; else 1, 2, 4 or 8 wavefronts sharing one row range */
     int reserved;         /* tail handling, for measurements: 0 = table; 1 = no tail balancing (no
-                             16-row pieces, no grouped launch); 2 + v = grouped launch of the table
-                             kernel with the last v row-block items of every XCD split by columns
-                             over a workgroup (v = 0: none split) */
+                             16-row pieces, no grouped launch); 2 + v + (h << 16) = grouped launch of
+                             the table kernel with the last v row-block items of every XCD split by
+                             columns over a workgroup (v = 0: none split), the last h - 1 of them
+                             also into two halves of 64 rows (h = 0: a quarter of v) */
 } km_launch_options;
 
 /* Message for the last error returned on the calling thread ("" if none). */

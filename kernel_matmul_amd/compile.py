@@ -111,7 +111,10 @@ class NativeModule:
         if self.defines.get("MATMUL_TAIL_BALANCE") == 0:
             options.reserved = 1
         elif self.defines.get("MATMUL_GROUP_TAIL") is not None:
-            options.reserved = 2 + int(self.defines["MATMUL_GROUP_TAIL"])
+            options.reserved = 2 + min(int(self.defines["MATMUL_GROUP_TAIL"]), 0xFFFF)
+            halves = self.defines.get("MATMUL_GROUP_TAIL_HALVES")
+            if halves is not None:
+                options.reserved += (min(int(halves), 0x3FFF) + 1) << 16
         rows = self.defines.get("MATMUL_ROWS_PER_WAVE")
         if rows is not None:
             options.rows_per_wave = int(rows)

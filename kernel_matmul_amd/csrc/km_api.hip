@@ -90,8 +90,12 @@ static int make_plan(const MatmulProblem& p, const km_launch_options* opt, Matmu
     int variant = opt ? opt->variant : KM_VARIANT_AUTO;
     plan->phase_split = 0;
     plan->group_tail = -1;
+    plan->group_tail_halves = -1;
     if (opt && opt->reserved >= 2) {
-        plan->group_tail = opt->reserved - 2;  // measurements: grouped launch with this many split items per XCD
+        // measurements: grouped launch with this many split items per XCD (low 16 bits); bits
+        // above: 0 = the usual share of them as two halves of 64 rows, else that count + 1
+        plan->group_tail = (opt->reserved - 2) & 0xffff;
+        plan->group_tail_halves = ((opt->reserved - 2) >> 16) - 1;
     }
     if (variant == KM_VARIANT_AUTO) {
         // Measured on gfx950 (n = 1e5 ... 1e6, batch 2 ... 8): with up to 16 rhs columns and enough
@@ -198,6 +202,11 @@ static int make_plan(const MatmulProblem& p, const km_launch_options* opt, Matmu
     }
     if (!(table && R == 8 && S == 1)) {
         plan->group_tail = -1;
+    }
+    // The very last of the split items also run as two halves of 64 rows (pieces of an eighth of
+    // an item; they repeat the column-side work).
+    if (plan->group_tail_halves < 0) {
+        plan->group_tail_halves = plan->group_tail > 0 ? plan->group_tail / 4 : 0;
     }
     return KM_OK;
 }
@@ -426,8 +435,9 @@ int km_matmul_describe(int kernel_type, int64_t num_batches, int64_t m, int64_t 
             if (plan.variant == KM_VARIANT_MFMA_F16 && plan.group_tail >= 0) {
                 snprintf(text, text_bytes,
                          "km::fwd_table_f16_grouped<%s>: 128 rows per wavefront, 4 wavefronts per workgroup, the "
-                         "last %lld items of each XCD split by columns over a workgroup",
-                         kt, plan.group_tail);
+                         "last %lld items of each XCD split by columns over a workgroup (the last %lld of them "
+                         "also into two halves of 64 rows)",
+                         kt, plan.group_tail, plan.group_tail_halves);
                 break;
             }
             snprintf(text, text_bytes, "%s<%s, G=%d, R=%d>: %d rows per wavefront, %d wavefront(s) per row range%s",

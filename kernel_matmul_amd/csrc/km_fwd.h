@@ -26,6 +26,8 @@ struct FwdArgs {
     int chunks_per_block;    // 128 / rows per workgroup
     int tail_items;          // per XCD: row-block items at the end that are dispatched last in pieces
                              // (direct kernel: 8 pieces of 16 rows; grouped table kernel: 4 column shares)
+    int tail_half_items;     // grouped table kernel: how many of these, the very last, are also cut
+                             // into two halves of 64 rows (two workgroups)
     const float* x1;
     const float* x2;
     const float* rhs;

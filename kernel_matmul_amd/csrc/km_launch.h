@@ -47,6 +47,7 @@ struct MatmulPlan {
     int phase_split;   // KM_VARIANT_BLOCK: spectral kernel in phase-split form
     long long group_tail;  // table kernel: >= 0 selects the grouped launch (workgroups of 4 wavefronts) with
                            // this many items per XCD split by columns at the end; < 0: one wavefront per workgroup
+    long long group_tail_halves;  // how many of those, the very last, also run as two halves of 64 rows
 };
 
 hipError_t launch_matmul(const MatmulProblem& p, const MatmulPlan& plan, hipStream_t stream);

@@ -911,15 +911,22 @@ __global__ void __launch_bounds__(64 * KM_GROUP_WAVES, 3) fwd_table_f16_grouped(
     const long long slot = blockIdx.x / KM_NUM_XCD;
     const long long main_items = a.items_per_xcd - a.tail_items;
     const long long main_groups = (main_items + KM_GROUP_WAVES - 1) / KM_GROUP_WAVES;
+    const long long whole_tail = a.tail_items - a.tail_half_items;
     const bool split = slot >= main_groups;
+    const bool halves = slot >= main_groups + whole_tail;
     long long local;
+    int half = 0;
     if (!split) {
         local = slot * KM_GROUP_WAVES + wave;
         if (local >= main_items) {
             return;
         }
-    } else {
+    } else if (!halves) {
         local = main_items + (slot - main_groups);
+    } else {
+        const long long u = slot - main_groups - whole_tail;
+        local = main_items + whole_tail + u / 2;
+        half = (int)(u % 2);
     }
     const long long item = (long long)xcd * a.items_per_xcd + local;
     if (item >= a.total_items) {
@@ -927,8 +934,13 @@ __global__ void __launch_bounds__(64 * KM_GROUP_WAVES, 3) fwd_table_f16_grouped(
     }
     int unused;
     const WaveView w = wave_view(a, item, 1, &unused);
-    fwd_table_f16_body<KT, 1, 8>(a, lds, w, w.row_block * KM_BLOCK_SIZE, split ? KM_GROUP_WAVES : 1,
-                                 split ? wave : 0, wave, true);
+    if (halves) {
+        fwd_table_f16_body<KT, 1, 4>(a, lds, w, w.row_block * KM_BLOCK_SIZE + 64 * half, KM_GROUP_WAVES, wave, wave,
+                                     true);
+    } else {
+        fwd_table_f16_body<KT, 1, 8>(a, lds, w, w.row_block * KM_BLOCK_SIZE, split ? KM_GROUP_WAVES : 1,
+                                     split ? wave : 0, wave, true);
+    }
 }
 
 // ---------------------------------------------------------------------------------------
@@ -1085,6 +1097,7 @@ void fill_fwd_args(const MatmulProblem& p, FwdArgs* args) {
     a.items_per_xcd = 0;
     a.chunks_per_block = 1;
     a.tail_items = 0;
+    a.tail_half_items = 0;
 }
 
 hipError_t launch_matmul(const MatmulProblem& p, const MatmulPlan& plan, hipStream_t stream) {
@@ -1104,6 +1117,7 @@ hipError_t launch_matmul(const MatmulProblem& p, const MatmulPlan& plan, hipStre
     }
     a.items_per_xcd = (a.total_items + KM_NUM_XCD - 1) / KM_NUM_XCD;
     a.tail_items = 0;
+    a.tail_half_items = 0;
     unsigned grid_x = (unsigned)(a.items_per_xcd * KM_NUM_XCD);
     const unsigned grid_y = (unsigned)((p.k + plan.k_chunk - 1) / plan.k_chunk);
     // Tail balancing (direct split-fp16 kernel, one wavefront per 128-row block): whatever does
@@ -1124,8 +1138,9 @@ hipError_t launch_matmul(const MatmulProblem& p, const MatmulPlan& plan, hipStre
     if (plan.variant == KM_VARIANT_MFMA_F16 && plan.group_tail >= 0 && plan.row_groups == 8 &&
         plan.col_splits == 1 && plan.k_chunk == 16 && p.kernel_type != KM_KERNEL_LOCALLY_PERIODIC) {
         a.tail_items = (int)(plan.group_tail < a.items_per_xcd ? plan.group_tail : a.items_per_xcd);
+        a.tail_half_items = (int)(plan.group_tail_halves < a.tail_items ? plan.group_tail_halves : a.tail_items);
         const long long main_groups = (a.items_per_xcd - a.tail_items + KM_GROUP_WAVES - 1) / KM_GROUP_WAVES;
-        const unsigned gx = (unsigned)((main_groups + a.tail_items) * KM_NUM_XCD);
+        const unsigned gx = (unsigned)((main_groups + a.tail_items + a.tail_half_items) * KM_NUM_XCD);
         const size_t table = (size_t)KM_GROUP_WAVES * KM_PHASE_TABLE_FLOATS * sizeof(float);
         static_assert(KM_GROUP_WAVES * 8 * 4 * 64 <= KM_GROUP_WAVES * KM_PHASE_TABLE_FLOATS,
                       "the reduction buffer of a split item must fit over the tables");

@@ -157,23 +157,28 @@ def test_forward_every_row_block_against_oracle(name, variant):
     assert np.all(err <= tol), (name, variant, worst, err[worst], expected[worst])
 
 
-@pytest.mark.parametrize("name,group_tail", [("headline", 0), ("headline", 97), ("headline", 10_000),
-                                             ("c2", 5), ("c3_rbf", 3)])
-def test_forward_grouped_launch_against_oracle(name, group_tail):
+@pytest.mark.parametrize("name,group_tail,halves", [("headline", 0, None), ("headline", 97, None),
+                                                    ("headline", 97, 0), ("headline", 97, 97),
+                                                    ("headline", 10_000, None), ("headline", 10_000, 0),
+                                                    ("c2", 5, None), ("c2", 5, 5), ("c3_rbf", 3, 2)])
+def test_forward_grouped_launch_against_oracle(name, group_tail, halves):
     """Workgroups of four wavefronts: full items one per wavefront, the last `group_tail` items of
-    every XCD split by columns between the four wavefronts of a workgroup (fixed-order sum)."""
+    every XCD split by columns between the four wavefronts of a workgroup (fixed-order sum), the
+    last `halves` of them (default: a quarter) also into two workgroups of 64 rows each."""
     kernel, n, batch, k, a, h = _build(name)
     op_args = (a["x"], a["x"], a["rhs"], a["params"], a["start"], a["end"])
     defines = MatmulSingleConfiguration(kernel).make_config(op_args)
     defines["MATMUL_VARIANT"] = "mfma_f16"
     defines["MATMUL_ROWS_PER_WAVE"] = 128
     defines["MATMUL_GROUP_TAIL"] = group_tail
+    if halves is not None:
+        defines["MATMUL_GROUP_TAIL_HALVES"] = halves
     out = load_native("matmul", defines).call(*op_args)
     again = load_native("matmul", defines).call(*op_args)
     assert torch.equal(out, again)  # fixed reduction order: reproducible
     expected = _forward_oracle(name, kernel, h)
     err = np.abs(out.cpu().double().numpy() - expected)
-    assert np.all(err <= 1e-5 + 1e-4 * np.abs(expected)), (name, group_tail, err.max())
+    assert np.all(err <= 1e-5 + 1e-4 * np.abs(expected)), (name, group_tail, halves, err.max())
 
 
 def test_split_fp16_error_against_fp32_mfma_on_headline():
