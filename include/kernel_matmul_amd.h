@@ -130,6 +130,13 @@ int km_matmul(int kernel_type, int batch_rank, const int64_t* batch_sizes, int64
 int km_matmul_describe(int kernel_type, int64_t num_batches, int64_t m, int64_t n, int64_t k,
                        const km_launch_options* options, char* text, size_t text_bytes);
 
+/* Which kernels and decomposition km_param_grad would pick for contiguous operands of this
+ * size (host only; nothing is launched): the feature form or the pairwise form, and the number
+ * of column shares per row block.  Like km_matmul_describe, it stands in for the reference's
+ * autotune report (kernel_matmul/native_function.py:56-69). */
+int km_param_grad_describe(int kernel_type, int64_t num_batches, int64_t m, int64_t c, char* text,
+                           size_t text_bytes);
+
 /* ------------------------------------------------------------------------------------
  * Hyper-parameter gradient of a bilinear form through the masked kernel matrix:
  *   grad[b,p] = d/d params[b,p]  sum_{(i,j) in mask} (sum_c left[b,i,c] right[b,j,c]) K[b,i,j]

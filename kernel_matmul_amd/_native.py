@@ -83,6 +83,9 @@ def load_library():
         + tensor * 6
         + [_vp, ctypes.POINTER(LaunchOptions), _vp]
     )
+    lib.km_param_grad_describe.restype = ctypes.c_int
+    lib.km_param_grad_describe.argtypes = [ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                                           ctypes.c_char_p, ctypes.c_size_t]
     lib.km_matmul_describe.restype = ctypes.c_int
     lib.km_matmul_describe.argtypes = [ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                                        ctypes.c_int64, _vp, ctypes.c_char_p, ctypes.c_size_t]
@@ -305,6 +308,16 @@ def matmul(kernel_type: str, x1: Tensor, x2: Tensor, rhs: Tensor, params: Tensor
     if status != 0:
         _raise(load_library(), status)
     return out
+
+
+def describe_param_grad(kernel_type: str, num_batches: int, m: int, c: int) -> str:
+    """Kernels and decomposition of the parameter gradient for this problem (C ABI: km_param_grad_describe)."""
+    lib = load_library()
+    text = ctypes.create_string_buffer(512)
+    status = lib.km_param_grad_describe(_kernel_id(kernel_type), num_batches, m, c, text, len(text))
+    if status != 0:
+        _raise(status, lib)
+    return text.value.decode()
 
 
 def describe_matmul(kernel_type: str, num_batches: int, m: int, n: int, k: int,

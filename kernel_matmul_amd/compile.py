@@ -121,11 +121,16 @@ class NativeModule:
         return options
 
     def describe(self, *args) -> str:
-        """Which kernel and decomposition ``call(*args)`` runs (matmul only; nothing is launched)."""
+        """Which kernel and decomposition ``call(*args)`` runs, as the library's launch tables
+        report it for matmul and the parameter gradients (nothing is launched)."""
+        if self.op in ("matmul_bwd", "bilinear_derivative"):
+            x1, left = args[0], args[2]
+            batches = 1
+            for size in x1.shape[:-1]:
+                batches *= size
+            return _native.describe_param_grad(self.kernel_type, batches, x1.shape[-1], left.shape[-1])
         if self.op != "matmul":
-            return {"matmul_bwd": "km::param_grad_partial + km::param_grad_reduce",
-                    "bilinear_derivative": "km::param_grad_partial + km::param_grad_reduce",
-                    "index": "km::index_kernel", "index_bwd": "km::index_bwd_terms + reduce",
+            return {"index": "km::index_kernel", "index_bwd": "km::index_bwd_terms + reduce",
                     "dense": "km::dense_kernel", "dense_bwd": "km::dense_bwd_partial + reduce"}[self.op]
         x1, x2, rhs = args[0], args[1], args[2]
         batches = 1

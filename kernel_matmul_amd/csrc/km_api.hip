@@ -396,6 +396,19 @@ int km_matmul(int kernel_type, int batch_rank, const int64_t* batch_sizes, int64
     return err == hipSuccess ? KM_OK : fail_hip(op, err);
 }
 
+int km_param_grad_describe(int kernel_type, int64_t num_batches, int64_t m, int64_t c, char* text,
+                           size_t text_bytes) {
+    const char* op = "km_param_grad_describe";
+    if (km_num_params(kernel_type) < 0) {
+        return fail(KM_ERR_UNSUPPORTED, "%s: unknown kernel type %d", op, kernel_type);
+    }
+    if (num_batches < 0 || m < 0 || c < 0 || text == nullptr || text_bytes == 0) {
+        return fail(KM_ERR_INVALID_ARGUMENT, "%s: invalid argument", op);
+    }
+    describe_param_grad(kernel_type, m, num_batches, c, text, text_bytes);
+    return KM_OK;
+}
+
 int km_matmul_describe(int kernel_type, int64_t num_batches, int64_t m, int64_t n, int64_t k,
                        const km_launch_options* options, char* text, size_t text_bytes) {
     const char* op = "km_matmul_describe";

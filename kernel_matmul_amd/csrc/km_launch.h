@@ -81,6 +81,9 @@ struct ParamGradProblem {
 long long param_grad_partials_per_batch(int64_t m, long long num_batches);
 // Same for the feature form of the first pass at vector width c (0 where the form does not apply).
 long long param_grad_feature_partials_per_batch(int kernel_type, int64_t m, long long num_batches, int64_t c);
+// Which kernels and decomposition launch_param_grad picks for contiguous operands of this size.
+void describe_param_grad(int kernel_type, int64_t m, long long num_batches, int64_t c, char* text,
+                         size_t text_bytes);
 hipError_t launch_param_grad(const ParamGradProblem& p, hipStream_t stream);
 
 struct IndexProblem {

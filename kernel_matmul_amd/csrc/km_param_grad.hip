@@ -16,6 +16,8 @@
 // Pass 2 (param_grad_reduce): one workgroup per batch item adds the partial rows in a
 // fixed order in fp64 and applies the chain rule back to the user parameters
 // (native/common/kernel_function.cuh:221-251).  No atomics: results are reproducible.
+#include <cstdio>
+
 #include "km_batch.h"
 #include "km_common.h"
 #include "km_fwd.h"
@@ -670,6 +672,26 @@ long long param_grad_feature_partials_per_batch(int kernel_type, int64_t m, long
     const long long row_blocks = (m + KM_BLOCK_SIZE - 1) / KM_BLOCK_SIZE;
     const long long chunks = row_blocks * (8 / f.R);
     return chunks * grad_col_splits(chunks * num_batches);
+}
+
+void describe_param_grad(int kernel_type, int64_t m, long long num_batches, int64_t c, char* text,
+                         size_t text_bytes) {
+    static const char* const kernels[] = {"rbf", "spectral", "locally_periodic"};
+    const FeaturePlan f = feature_plan(kernel_type, c);
+    const long long row_blocks = (m + KM_BLOCK_SIZE - 1) / KM_BLOCK_SIZE;
+    const int splits = grad_col_splits(row_blocks * num_batches);
+    if (f.GE > 0) {
+        snprintf(text, text_bytes,
+                 "km::param_grad_features<%s, GE=%d, R=%d, TL=%d> (feature form; per-item pairwise fallback) + "
+                 "km::param_grad_reduce: 128 rows per wavefront, %d column share(s) per row block",
+                 kernels[kernel_type], f.GE, f.R, f.TL, splits);
+    } else {
+        const int tl = c <= 4 ? 1 : (c <= 8 ? 2 : (c <= 16 ? 4 : 0));
+        snprintf(text, text_bytes,
+                 "km::param_grad_partial<%s, TL=%d> (pairwise form) + km::param_grad_reduce: 128 rows per "
+                 "wavefront, %d column share(s) per row block",
+                 kernels[kernel_type], tl, splits);
+    }
 }
 
 template <int KT, int GE, int R, int TL>

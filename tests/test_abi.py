@@ -85,3 +85,20 @@ def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(_native, "LIB_PATH", "/nonexistent/libkernel_matmul_amd.so")
     with pytest.raises(RuntimeError, match="native library not found"):
         _native.load_library()
+
+
+def test_launch_descriptions_without_a_gpu():
+    """km_matmul_describe / km_param_grad_describe report the launch tables' choices (host only)."""
+    text = _native.describe_matmul("spectral", 8, 100_000, 100_000, 16, None)
+    assert "fwd_table_f16_grouped<spectral>" in text and "128 rows per wavefront" in text
+    assert "fwd_mfma_f16<spectral" in _native.describe_matmul("spectral", 8, 1_000_000, 1_000_000, 32, None)
+    assert "fwd_block<rbf" in _native.describe_matmul("rbf", 8, 1_000_000, 1_000_000, 16, None)
+    # narrow vectors: feature form; wide ones and the locally periodic kernel: pairwise form
+    assert "param_grad_features<spectral, GE=2" in _native.describe_param_grad("spectral", 16, 100_000, 4)
+    assert "param_grad_partial<spectral, TL=2>" in _native.describe_param_grad("spectral", 2, 50_000, 8)
+    assert "param_grad_features<rbf, GE=2" in _native.describe_param_grad("rbf", 2, 50_000, 10)
+    assert "param_grad_partial<locally_periodic" in _native.describe_param_grad("locally_periodic", 2, 5_000, 3)
+    lib = _native.load_library()
+    buf = ctypes.create_string_buffer(16)
+    assert lib.km_param_grad_describe(7, 1, 128, 4, buf, len(buf)) == -2
+    assert lib.km_param_grad_describe(1, 1, 128, 4, None, 0) == -1
