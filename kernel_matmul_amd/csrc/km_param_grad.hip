@@ -88,11 +88,41 @@ __device__ __forceinline__ void pairwise_item(const GradArgs& a, const float* __
 
     float acc[KM_MAX_PARAMS] = {0.0f, 0.0f, 0.0f, 0.0f};
 
+    // Operands of a chunk of 16 columns: x2 of column n0 + li and, with the left operand in
+    // registers, the right operand's values (column n0 + li, vector column 4 t + kk), zero outside
+    // the range.  They are requested one chunk ahead.
+    auto load_chunk = [&](int n0, float* x2v, float (&rv)[TLR]) {
+        const int col = n0 + li;
+        const int col_c = min(col, col_end - 1);
+        *x2v = x2[(long long)col_c * a.x2_s];
+        if (TL > 0) {
+#pragma unroll
+            for (int t = 0; t < TLR; t++) {
+                const int cc = 4 * t + kk;
+                rv[t] = (col < col_end && cc < a.c)
+                            ? right[(long long)col_c * a.right_s0 + (long long)cc * a.right_s1]
+                            : 0.0f;
+            }
+        }
+    };
+    float x2_next = 0.0f, rv_next[TLR];
+    if (col_begin < col_end) {
+        load_chunk(col_begin, &x2_next, rv_next);
+    }
+
     for (int n0 = col_begin; n0 < col_end; n0 += 16) {
         const int col = n0 + li;
         const bool col_ok = col < col_end;
         const int col_c = min(col, col_end - 1);
-        const float x2v = x2[(long long)col_c * a.x2_s];
+        const float x2v = x2_next;
+        float rvs[TLR];
+#pragma unroll
+        for (int t = 0; t < TLR; t++) {
+            rvs[t] = rv_next[t];
+        }
+        if (n0 + 16 < col_end) {
+            load_chunk(n0 + 16, &x2_next, rv_next);
+        }
 
         float4v coef[R];
 #pragma unroll
@@ -103,13 +133,9 @@ __device__ __forceinline__ void pairwise_item(const GradArgs& a, const float* __
         if (TL > 0) {
 #pragma unroll
             for (int t = 0; t < TLR; t++) {
-                const int cc = 4 * t + kk;
-                const float rv = (col_ok && cc < a.c)
-                                     ? right[(long long)col_c * a.right_s0 + (long long)cc * a.right_s1]
-                                     : 0.0f;
 #pragma unroll
                 for (int r = 0; r < R; r++) {
-                    coef[r] = __builtin_amdgcn_mfma_f32_16x16x4f32(lreg[r][t], rv, coef[r], 0, 0, 0);
+                    coef[r] = __builtin_amdgcn_mfma_f32_16x16x4f32(lreg[r][t], rvs[t], coef[r], 0, 0, 0);
                 }
             }
         } else {
