@@ -161,6 +161,23 @@ static int make_plan(const MatmulProblem& p, const km_launch_options* opt, Matmu
             R /= 2;
         }
     }
+    // Register budget of the split-fp16 kernels: their operand buffers and accumulators grow with
+    // the number of rhs column groups, so wide rhs tiles get fewer row groups per wavefront (no
+    // spills, at least two wavefronts per SIMD: G * R = 16 takes 191 to 250 VGPRs).  Measured:
+    // 4 row groups instead of 2 at k = 64 save 25-28 % (n = 1e5, batch 8: 228 against 305 us),
+    // 8 instead of 4 at k = 32 save 7-12 % (n = 1e6: 1.30 against 1.39 ms).
+    if (variant == KM_VARIANT_MFMA_F16 || variant == KM_VARIANT_MFMA_F16_DIRECT) {
+        const int groups = phase_split ? 2 * G : G;
+        const int max_r = groups == 1 ? 8 : (groups == 2 ? 8 : (groups == 4 ? 4 : 2));
+        if (R > max_r) {
+            R = max_r;
+        }
+    }
+    // Kernels at 2 wavefronts per SIMD (the direct kernel at G * R = 16) want 2048 wavefronts
+    // before column ranges stop being shared (rbf, n = 65536, k = 64, batch 1: 45.4 us with two
+    // wavefronts per row range against 52.9 us with one); the others 1024.
+    const bool two_per_simd = variant == KM_VARIANT_MFMA_F16_DIRECT && G * R >= 16;
+    const long long wave_target = two_per_simd ? 2 * TARGET_WAVES : TARGET_WAVES;
     int S = 1;
     if (opt && opt->col_splits != 0) {
         S = opt->col_splits;
@@ -168,17 +185,8 @@ static int make_plan(const MatmulProblem& p, const km_launch_options* opt, Matmu
             return fail(KM_ERR_INVALID_ARGUMENT, "km_matmul: col_splits must be 1, 2, 4 or 8");
         }
     } else {
-        while (S < 8 && base * (8 / R) * S < TARGET_WAVES) {
+        while (S < 8 && base * (8 / R) * S < wave_target) {
             S *= 2;
-        }
-    }
-    // Register budget of the split-fp16 kernel: its operand buffers grow with G, so wide rhs
-    // tiles get fewer row groups per wavefront (no spills, at least two wavefronts per SIMD).
-    if (variant == KM_VARIANT_MFMA_F16 || variant == KM_VARIANT_MFMA_F16_DIRECT) {
-        const int groups = phase_split ? 2 * G : G;
-        const int max_r = groups == 1 ? 8 : (groups == 2 ? (phase_split ? 8 : 4) : (groups == 4 ? (phase_split ? 4 : 2) : 2));
-        if (R > max_r) {
-            R = max_r;
         }
     }
     // LDS per workgroup must stay within 64 KiB: the cross-wavefront reduction buffer takes

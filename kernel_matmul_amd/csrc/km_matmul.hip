@@ -1023,7 +1023,7 @@ static hipError_t launch_mfma(const FwdArgs& a, int variant, int S, unsigned gx,
     } else if (variant == KM_VARIANT_MFMA_F16_DIRECT) {
         // Wide rhs tiles with many row groups exceed the register file; the launch table never
         // picks them.
-        if constexpr (G * R <= 8) {
+        if constexpr (G * R <= 16) {
             hipLaunchKernelGGL((fwd_mfma_f16<KT, G, R, G == 1>), dim3(gx, gy, 1), dim3(64 * S, 1, 1), lds, stream, a);
         } else {
             return hipErrorInvalidConfiguration;
