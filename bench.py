@@ -80,6 +80,8 @@ def make_workload(name: str, batch_override=None):
         params = 1.0 + 0.01 * torch.randn(*bshape, 2, generator=g)
     elif w["kernel"] == "spectral":
         params = torch.stack([u(0.5, 2.0), u(0.05, 0.5), u(0.5, 2.0)], dim=-1)
+    elif w["kernel"] == "locally_periodic":
+        params = torch.stack([u(0.5, 2.0), u(0.5, 2.0), u(0.5, 2.0), u(0.5, 2.0)], dim=-1)
     else:
         params = torch.stack([torch.ones(bshape), torch.ones(bshape)], dim=-1)
     rhs = torch.randn(n, w["k"], generator=g)

@@ -59,8 +59,8 @@ typedef struct km_launch_options {
                              4 = split-fp16 MFMA with the kernel evaluated directly per pair,
                              5 = split-fp16 MFMA with the rhs operand prepared once per workgroup
                              of four row blocks (rows_per_wave / col_splits must stay 0).
-                             The table picks 5 for large rbf / locally periodic problems with at
-                             most 16 rhs columns and 3 otherwise. */
+                             The table picks 5 for large locally periodic problems with at most
+                             16 rhs columns and 3 otherwise. */
     int rows_per_wave;    /* 0 = table; else 16, 32, 64 or 128 rows of x1 per wavefront */
     int col_splits;       /* 0 = table; else 1, 2, 4 or 8 wavefronts sharing one row range */
     int reserved;         /* tail handling, for measurements: 0 = table; 1 = no tail balancing (no

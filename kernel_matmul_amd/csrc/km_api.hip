@@ -98,13 +98,13 @@ static int make_plan(const MatmulProblem& p, const km_launch_options* opt, Matmu
         plan->group_tail_halves = ((opt->reserved - 2) >> 16) - 1;
     }
     if (variant == KM_VARIANT_AUTO) {
-        // Measured on gfx950 (n = 1e5 ... 1e6, batch 2 ... 8): with up to 16 rhs columns and enough
-        // row blocks to fill the device several times, sharing the rhs operand between four row
-        // blocks wins for the rbf (7 %) and locally periodic (12-18 %) kernels; the phase-split
-        // spectral kernel and everything with wider rhs or fewer row blocks is faster with one
-        // wavefront per row block.
+        // Measured on gfx950 (n = 1e5, k = 16): for the locally periodic kernel with enough row
+        // blocks to fill the device several times, sharing the rhs operand between four row
+        // blocks wins (batch 8: 133 against 154 us; batch 2: 52 against 49 us, hence the
+        // threshold); rbf and spectral kernels are faster through the column tables with one
+        // wavefront per row block (rbf, batch 8: 77 against 86 us; batch 64: 494 against 578 us).
         const long long row_blocks = (p.m + KM_BLOCK_SIZE - 1) / KM_BLOCK_SIZE;
-        const bool shared = p.kernel_type != KM_KERNEL_SPECTRAL && p.k <= 16 &&
+        const bool shared = p.kernel_type == KM_KERNEL_LOCALLY_PERIODIC && p.k <= 16 &&
                             row_blocks * p.num_batches >= BLOCK_VARIANT_MIN_ITEMS &&
                             !(opt && (opt->rows_per_wave != 0 || opt->col_splits > 1));
         variant = shared ? KM_VARIANT_BLOCK : KM_VARIANT_MFMA_F16;

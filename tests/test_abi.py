@@ -92,7 +92,8 @@ def test_launch_descriptions_without_a_gpu():
     text = _native.describe_matmul("spectral", 8, 100_000, 100_000, 16, None)
     assert "fwd_table_f16_grouped<spectral>" in text and "128 rows per wavefront" in text
     assert "fwd_mfma_f16<spectral" in _native.describe_matmul("spectral", 8, 1_000_000, 1_000_000, 32, None)
-    assert "fwd_block<rbf" in _native.describe_matmul("rbf", 8, 1_000_000, 1_000_000, 16, None)
+    assert "fwd_table_f16_grouped<rbf>" in _native.describe_matmul("rbf", 8, 1_000_000, 1_000_000, 16, None)
+    assert "fwd_block<locally_periodic" in _native.describe_matmul("locally_periodic", 8, 1_000_000, 1_000_000, 16, None)
     # narrow vectors: feature form; wide ones and the locally periodic kernel: pairwise form
     assert "param_grad_features<spectral, GE=2" in _native.describe_param_grad("spectral", 16, 100_000, 4)
     assert "param_grad_partial<spectral, TL=2>" in _native.describe_param_grad("spectral", 2, 50_000, 8)
