@@ -184,6 +184,29 @@ static int make_plan(const MatmulProblem& p, const km_launch_options* opt, Matmu
         if (S != 1 && S != 2 && S != 4 && S != 8) {
             return fail(KM_ERR_INVALID_ARGUMENT, "km_matmul: col_splits must be 1, 2, 4 or 8");
         }
+    } else if (table && !two_per_simd) {
+        // Table kernels: the share count that leaves the fullest SIMD the least work,
+        // ceil(wavefronts / 1024) pieces of 1 / S of an item at 8 % of overhead per doubling
+        // (n = 20000, batch 4: 1256 wavefronts of 64 rows leave 232 SIMDs with two of them, 31 us;
+        // two shares each, three quarter-size pieces at most, 26 us; with 1564 wavefronts
+        // (n = 50000, batch 2) two shares would make it four pieces: 33 against 28 us).
+        const long long waves = base * (8 / R);
+        double best = 0.0;
+        for (int s = 1; s <= 8; s *= 2) {
+            const long long pieces = (waves * s + TARGET_WAVES - 1) / TARGET_WAVES;
+            double overhead = 1.0;
+            for (int t = 1; t < s; t *= 2) {
+                overhead *= 1.08;
+            }
+            const double cost = (double)pieces / s * overhead;
+            if (s == 1 || cost < best * 0.97) {
+                best = cost;
+                S = s;
+            }
+            if (waves * s >= 4 * TARGET_WAVES) {
+                break;
+            }
+        }
     } else {
         while (S < 8 && base * (8 / R) * S < wave_target) {
             S *= 2;
