@@ -253,14 +253,18 @@ __global__ void __launch_bounds__(64) param_grad_partial(const GradArgs a) {
 #define KM_GF_CHUNK 256
 #define KM_GF_MAX_FEATURES 6
 #define KM_GF_MAX_WIDTH 10 /* widest vector the feature form takes */
-#define KM_GF_TABLE_FLOATS \
-    ((1 + KM_GF_MAX_FEATURES) * KM_GF_CHUNK + KM_GF_CHUNK / 8 + 3 * KM_BLOCK_SIZE + KM_BLOCK_SIZE * KM_GF_MAX_WIDTH)
+/* column tables of a chunk (b, features, reference points) or, in the epilogue, the row weights */
+#define KM_GF_HEAD_FLOATS (KM_BLOCK_SIZE * KM_GF_MAX_FEATURES * 3)
+#define KM_GF_TABLE_FLOATS (KM_GF_HEAD_FLOATS + KM_BLOCK_SIZE * KM_GF_MAX_WIDTH)
 #define KM_GF_HMAX 12.0f
 #define KM_GF_GMAX 48.0f
 
 template <int KT, int GE, int R, int TL>
 __global__ void __launch_bounds__(64, 2) param_grad_features(const GradArgs a) {
     static_assert(KT == KM_KERNEL_RBF || KT == KM_KERNEL_SPECTRAL, "feature form: rbf or spectral");
+    static_assert(R == 8, "128 rows per item (row weights: two rows per lane)");
+    static_assert((1 + KM_GF_MAX_FEATURES) * KM_GF_CHUNK + KM_GF_CHUNK / 8 <= KM_GF_HEAD_FLOATS,
+                  "the column tables must fit in front of the staged rows of left");
     constexpr bool PHASE = KT == KM_KERNEL_SPECTRAL;
     constexpr int NF = PHASE ? 6 : 3;
     constexpr int CH = KM_GF_CHUNK;
@@ -269,8 +273,8 @@ __global__ void __launch_bounds__(64, 2) param_grad_features(const GradArgs a) {
     float* tab_b = lds;                    // (x2 - r) s per column, r: reference of its 8 columns
     float* tab_f = lds + CH;               // [NF][CH] column features times 2^(-b^2)
     float* tab_ref = lds + (1 + KM_GF_MAX_FEATURES) * CH;
-    float* tab_rows = tab_ref + CH / 8;    // [3][16 R]: cos A, sin A, h per row (epilogue)
-    float* tab_left = tab_rows + 3 * KM_BLOCK_SIZE;  // [16 R][c]: this item's rows of `left` (epilogue)
+    // (the epilogue's row weights, [16 R][NF][3], later overlay everything up to here)
+    float* tab_left = lds + KM_GF_HEAD_FLOATS;  // [16 R][c]: this item's rows of `left` (epilogue)
 
     GradItem g;
     if (!grad_item(a, 16 * R, 32, &g)) {
@@ -527,59 +531,69 @@ __global__ void __launch_bounds__(64, 2) param_grad_features(const GradArgs a) {
         return;
     }
 
-    // Rows: cos A, sin A and h, by the lanes that hold the coordinates (A layout), read back in
-    // the D layout (rows 16 r + 4 kk + v).
-    if (kk == 0) {
+    // Row weights of the three sums for every feature, tab_w[row][feature][3], over the column
+    // tables (all reads of those are done).  With pw the power of g in the feature and cB / sB its
+    // phase factor, (h - g)^2 contributes h^2, -2 h, 1 and (h - g) contributes h, -1, 0 for
+    // pw = 0, 1, 2; cos(A - B) = cA cB + sA sB puts cA on the cB features and sA on the sB ones,
+    // sin(A - B) = sA cB - cA sB puts sA and -cA there.  Each lane forms the weights of two
+    // rows (lane and lane + 64; it holds their coordinates in the A layout: row 16 r + lane % 16).
+    float* tab_w = lds;
+    {
+        const float xa = kk == 0 ? x1v[0] : (kk == 1 ? x1v[1] : (kk == 2 ? x1v[2] : x1v[3]));
+        const float xb = kk == 0 ? x1v[4] : (kk == 1 ? x1v[5] : (kk == 2 ? x1v[6] : x1v[7]));
 #pragma unroll
-        for (int r = 0; r < R; r++) {
-            float ca = 1.0f, sa = 0.0f;
+        for (int half = 0; half < 2; half++) {
+            const float xr = half == 0 ? xa : xb;
+            float* w = tab_w + (size_t)(64 * half + lane) * (NF * 3);
+            const float h = (xr - c0) * kc.s;
+            const float h2 = h * h;
             if (PHASE) {
-                const float th = phase_rev(kc.f, x1v[r], c0);
-                ca = __builtin_amdgcn_cosf(th);
-                sa = __builtin_amdgcn_sinf(th);
+                const float th = phase_rev(kc.f, xr, c0);
+                const float ca = __builtin_amdgcn_cosf(th);
+                const float sa = __builtin_amdgcn_sinf(th);
+                const float m2h = -2.0f * h;
+                w[0] = ca * h2;   w[1] = sa * h;    w[2] = ca;     // cB
+                w[3] = sa * h2;   w[4] = -ca * h;   w[5] = sa;     // sB
+                w[6] = ca * m2h;  w[7] = -sa;       w[8] = 0.0f;   // cB g
+                w[9] = sa * m2h;  w[10] = ca;       w[11] = 0.0f;  // sB g
+                w[12] = ca;       w[13] = 0.0f;     w[14] = 0.0f;  // cB g^2
+                w[15] = sa;       w[16] = 0.0f;     w[17] = 0.0f;  // sB g^2
+            } else {
+                w[0] = h2;          w[1] = 1.0f;  w[2] = 0.0f;  // 1
+                w[3] = -2.0f * h;   w[4] = 0.0f;  w[5] = 0.0f;  // g
+                w[6] = 1.0f;        w[7] = 0.0f;  w[8] = 0.0f;  // g^2
             }
-            tab_rows[16 * r + li] = ca;
-            tab_rows[16 * R + 16 * r + li] = sa;
-            tab_rows[32 * R + 16 * r + li] = (x1v[r] - c0) * kc.s;
         }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
+    // Accumulators in the D layout: rows 16 r + 4 kk + v, operand column (feature, vector column)
+    // of the lane.  Every value times its row's `left` entry and the row weights of its feature.
     float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f;
-    int pw[GE];        // power of g in the lane's feature of group ge
-    bool odd[GE];      // sin B (odd) or cos B (even) feature
     float unscale[GE];
+    const float* wlane[GE];
+    const float* llane[GE];
 #pragma unroll
     for (int ge = 0; ge < GE; ge++) {
-        pw[ge] = PHASE ? (feat[ge] >> 1) : feat[ge];
-        odd[ge] = PHASE && (feat[ge] & 1);
         unscale[ge] = used[ge] ? __builtin_ldexpf(1.0f, -shift[ge] - KS) : 0.0f;
+        wlane[ge] = tab_w + (4 * kk) * (NF * 3) + feat[ge] * 3;
+        llane[ge] = tab_left + (4 * kk) * a.c + vcol[ge];
     }
 #pragma unroll
     for (int r = 0; r < R; r++) {
-        const float4v ca4 = *(const float4v*)(tab_rows + 16 * r + 4 * kk);
-        const float4v sa4 = *(const float4v*)(tab_rows + 16 * R + 16 * r + 4 * kk);
-        const float4v h4 = *(const float4v*)(tab_rows + 32 * R + 16 * r + 4 * kk);
 #pragma unroll
         for (int ge = 0; ge < GE; ge++) {
 #pragma unroll
             for (int v = 0; v < 4; v++) {
-                const float lv = tab_left[(16 * r + 4 * kk + v) * a.c + vcol[ge]];
+                const float* w = wlane[ge] + (16 * r + v) * (NF * 3);
+                const float lv = llane[ge][(16 * r + v) * a.c];
                 const float val = acc[r][ge][v] * unscale[ge] * lv;
-                const float h = h4[v];
-                const float poly = pw[ge] == 0 ? h * h : (pw[ge] == 1 ? -2.0f * h : 1.0f);  // of (h - g)^2
+                s0 = __builtin_fmaf(w[0], val, s0);
+                s1 = __builtin_fmaf(w[1], val, s1);
                 if (PHASE) {
-                    const float base = odd[ge] ? sa4[v] : ca4[v];   // cos(A - B): cA cB + sA sB
-                    const float alt = odd[ge] ? -ca4[v] : sa4[v];   // sin(A - B): sA cB - cA sB
-                    const float lin = pw[ge] == 0 ? h : (pw[ge] == 1 ? -1.0f : 0.0f);  // of (h - g)
-                    s0 = __builtin_fmaf(base * poly, val, s0);
-                    s1 = __builtin_fmaf(alt * lin, val, s1);
-                    s2 = __builtin_fmaf(pw[ge] == 0 ? base : 0.0f, val, s2);
-                } else {
-                    s0 = __builtin_fmaf(poly, val, s0);
-                    s1 = __builtin_fmaf(pw[ge] == 0 ? 1.0f : 0.0f, val, s1);
+                    s2 = __builtin_fmaf(w[2], val, s2);
                 }
             }
         }
