@@ -270,7 +270,7 @@ __global__ void __launch_bounds__(64, 2) param_grad_features(const GradArgs a) {
     constexpr int CH = KM_GF_CHUNK;
     constexpr int KS = KM_TABLE_KSCALE_LOG2;
     extern __shared__ float lds[];
-    float* tab_b = lds;                    // (x2 - r) s per column, r: reference of its 8 columns
+    float* tab_b = lds;                    // 2 (x2 - r) s per column, r: reference of its 8 columns
     float* tab_f = lds + CH;               // [NF][CH] column features times 2^(-b^2)
     float* tab_ref = lds + (1 + KM_GF_MAX_FEATURES) * CH;
     // (the epilogue's row weights, [16 R][NF][3], later overlay everything up to here)
@@ -390,7 +390,7 @@ __global__ void __launch_bounds__(64, 2) param_grad_features(const GradArgs a) {
                 p0 = wgt * __builtin_amdgcn_cosf(th);
                 p1 = wgt * __builtin_amdgcn_sinf(th);
             }
-            tab_b[q] = b;
+            tab_b[q] = b + b;  // the form the rows' exponent takes it in
             if (PHASE) {
                 tab_f[0 * CH + q] = p0;
                 tab_f[1 * CH + q] = p1;
@@ -503,11 +503,10 @@ __global__ void __launch_bounds__(64, 2) param_grad_features(const GradArgs a) {
             for (int r = 0; r < R; r++) {
                 half2v h2[4], l2[4];
                 const float av = (x1v[r] - ref) * kc.s;
-                const float ra = av + av;
                 const float rb = __builtin_fmaf(-av, av, (float)KS);
 #pragma unroll
                 for (int t = 0; t < 4; t++) {
-                    separable_pair_f16(ra, rb, bv[2 * t], bv[2 * t + 1], kc.one, &h2[t], &l2[t]);
+                    separable_pair_f16(av, rb, bv[2 * t], bv[2 * t + 1], kc.one, &h2[t], &l2[t]);
                 }
                 const half8v ahi = join_half2x4(h2);
                 const half8v alo = join_half2x4(l2);
