@@ -250,11 +250,11 @@ __global__ void __launch_bounds__(64) param_grad_partial(const GradArgs a) {
 // of the fp16 operands) and every chunk of columns admits the separable exponent; an item that
 // fails any of these is redone in the pairwise form.
 // ---------------------------------------------------------------------------------------
-#define KM_GF_CHUNK 256
+#define KM_GF_CHUNK 512
 #define KM_GF_MAX_FEATURES 6
 #define KM_GF_MAX_WIDTH 10 /* widest vector the feature form takes */
 /* column tables of a chunk (b, features, reference points) or, in the epilogue, the row weights */
-#define KM_GF_HEAD_FLOATS (KM_BLOCK_SIZE * KM_GF_MAX_FEATURES * 3)
+#define KM_GF_HEAD_FLOATS ((1 + KM_GF_MAX_FEATURES) * KM_GF_CHUNK + KM_GF_CHUNK / 8)
 #define KM_GF_TABLE_FLOATS (KM_GF_HEAD_FLOATS + KM_BLOCK_SIZE * KM_GF_MAX_WIDTH)
 #define KM_GF_HMAX 12.0f
 #define KM_GF_GMAX 48.0f
@@ -263,8 +263,8 @@ template <int KT, int GE, int R, int TL>
 __global__ void __launch_bounds__(64, 2) param_grad_features(const GradArgs a) {
     static_assert(KT == KM_KERNEL_RBF || KT == KM_KERNEL_SPECTRAL, "feature form: rbf or spectral");
     static_assert(R == 8, "128 rows per item (row weights: two rows per lane)");
-    static_assert((1 + KM_GF_MAX_FEATURES) * KM_GF_CHUNK + KM_GF_CHUNK / 8 <= KM_GF_HEAD_FLOATS,
-                  "the column tables must fit in front of the staged rows of left");
+    static_assert(KM_BLOCK_SIZE * KM_GF_MAX_FEATURES * 3 <= KM_GF_HEAD_FLOATS,
+                  "the row weights must fit in front of the staged rows of left");
     constexpr bool PHASE = KT == KM_KERNEL_SPECTRAL;
     constexpr int NF = PHASE ? 6 : 3;
     constexpr int CH = KM_GF_CHUNK;
@@ -359,7 +359,7 @@ __global__ void __launch_bounds__(64, 2) param_grad_features(const GradArgs a) {
             for (int i = 0; i < CH / 64; i++) {
                 xq[i] = x2c[(unsigned long long)(unsigned)min(lane + 64 * i, last) * x2_stride];
             }
-            const float ref_own = x2c[(unsigned long long)(unsigned)min(8 * (lane & 31) + 4, last) * x2_stride];
+            const float ref_own = x2c[(unsigned long long)(unsigned)min(8 * (lane & (CH / 8 - 1)) + 4, last) * x2_stride];
 #pragma unroll
             for (int i = 0; i < CH / 64; i++) {
                 tab_b[lane + 64 * i] = xq[i];
