@@ -263,7 +263,7 @@ template <int KT, int GE, int R, int TL>
 __global__ void __launch_bounds__(64, 2) param_grad_features(const GradArgs a) {
     static_assert(KT == KM_KERNEL_RBF || KT == KM_KERNEL_SPECTRAL, "feature form: rbf or spectral");
     static_assert(R == 8, "128 rows per item (row weights: two rows per lane)");
-    static_assert(KM_BLOCK_SIZE * (KM_GF_MAX_FEATURES * 3 + 1) <= KM_GF_HEAD_FLOATS,
+    static_assert(KM_BLOCK_SIZE * KM_GF_MAX_FEATURES * 3 <= KM_GF_HEAD_FLOATS,
                   "the row weights must fit in front of the staged rows of left");
     constexpr bool PHASE = KT == KM_KERNEL_SPECTRAL;
     constexpr int NF = PHASE ? 6 : 3;
@@ -530,21 +530,20 @@ __global__ void __launch_bounds__(64, 2) param_grad_features(const GradArgs a) {
         return;
     }
 
-    // Row weights of the three sums for every feature, tab_w[row][feature][3] (rows padded to an odd stride), over the column
+    // Row weights of the three sums for every feature, tab_w[row][feature][3], over the column
     // tables (all reads of those are done).  With pw the power of g in the feature and cB / sB its
     // phase factor, (h - g)^2 contributes h^2, -2 h, 1 and (h - g) contributes h, -1, 0 for
     // pw = 0, 1, 2; cos(A - B) = cA cB + sA sB puts cA on the cB features and sA on the sB ones,
     // sin(A - B) = sA cB - cA sB puts sA and -cA there.  Each lane forms the weights of two
     // rows (lane and lane + 64; it holds their coordinates in the A layout: row 16 r + lane % 16).
     float* tab_w = lds;
-    constexpr int WS = NF * 3 + 1;  // floats per row (odd: the lanes' rows fall into distinct banks)
     {
         const float xa = kk == 0 ? x1v[0] : (kk == 1 ? x1v[1] : (kk == 2 ? x1v[2] : x1v[3]));
         const float xb = kk == 0 ? x1v[4] : (kk == 1 ? x1v[5] : (kk == 2 ? x1v[6] : x1v[7]));
 #pragma unroll
         for (int half = 0; half < 2; half++) {
             const float xr = half == 0 ? xa : xb;
-            float* w = tab_w + (size_t)(64 * half + lane) * WS;
+            float* w = tab_w + (size_t)(64 * half + lane) * (NF * 3);
             const float h = (xr - c0) * kc.s;
             const float h2 = h * h;
             if (PHASE) {
@@ -578,7 +577,7 @@ __global__ void __launch_bounds__(64, 2) param_grad_features(const GradArgs a) {
 #pragma unroll
     for (int ge = 0; ge < GE; ge++) {
         unscale[ge] = used[ge] ? __builtin_ldexpf(1.0f, -shift[ge] - KS) : 0.0f;
-        wlane[ge] = tab_w + (4 * kk) * WS + feat[ge] * 3;
+        wlane[ge] = tab_w + (4 * kk) * (NF * 3) + feat[ge] * 3;
         llane[ge] = tab_left + (4 * kk) * a.c + vcol[ge];
     }
 #pragma unroll
@@ -587,7 +586,7 @@ __global__ void __launch_bounds__(64, 2) param_grad_features(const GradArgs a) {
         for (int ge = 0; ge < GE; ge++) {
 #pragma unroll
             for (int v = 0; v < 4; v++) {
-                const float* w = wlane[ge] + (16 * r + v) * WS;
+                const float* w = wlane[ge] + (16 * r + v) * (NF * 3);
                 const float lv = llane[ge][(16 * r + v) * a.c];
                 const float val = acc[r][ge][v] * unscale[ge] * lv;
                 s0 = __builtin_fmaf(w[0], val, s0);
