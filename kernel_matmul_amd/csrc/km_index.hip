@@ -4,8 +4,10 @@
 //               (native/index/index.cu:12-101 of the reference).
 //   index_bwd : grad[b,p] = d/d params[b,p] sum_{q : batch(q) = b} out_grad[q] * out[q]
 //               (native/index_bwd/index_bwd.cu:12-112).  Pass 1 writes the derivative terms of
-//               every entry and the batch item it belongs to; pass 2 lets one workgroup per
-//               batch item add its entries in a fixed order in fp64 and applies the chain rule.
+//               every entry and the batch item it belongs to, and per block of 256 entries their
+//               fp64 sums and whether they all belong to one batch item; pass 2 lets one
+//               workgroup per batch item add its blocks' sums (the entries themselves only for
+//               blocks that mix batch items) in a fixed order and applies the chain rule.
 #include "km_common.h"
 #include "km_launch.h"
 
@@ -43,8 +45,11 @@ struct IndexArgs {
     // index_bwd only
     const float* out_grad;
     IndexStrides out_grad_strides;
-    float* terms;     // [total][KM_MAX_PARAMS]
-    int* owner;       // [total] flat batch item of the entry, -1 if it contributes nothing
+    float* terms;     // [total][KM_MAX_PARAMS] (written for the blocks that mix batch items)
+    int* owner;       // [total] flat batch item of the entry, -1 if it contributes nothing (likewise)
+    int* block_owner;    // [blocks of 256 entries] the one batch item of the block's entries, -1: none
+                         // contributes, -2: several batch items (the per-entry arrays decide)
+    double* block_sum;   // [blocks][KM_MAX_PARAMS] sums of the block's terms (fixed order)
     long long num_batches;
     float* grad;      // [num_batches][P]
 };
@@ -136,23 +141,55 @@ __global__ void __launch_bounds__(256) index_kernel(const IndexArgs a) {
 
 template <int KT>
 __global__ void __launch_bounds__(256) index_bwd_terms(const IndexArgs a) {
+    __shared__ double sh_sum[KM_MAX_PARAMS][256];
+    __shared__ int sh_lo[256], sh_hi[256];
     const long long q = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (q >= a.total) {
-        return;
-    }
-    const Entry en = decode_entry(a, q);
     float acc[KM_MAX_PARAMS] = {0.0f, 0.0f, 0.0f, 0.0f};
     int owner = -1;
-    if (en.inside) {
-        const KernelConsts kc = make_consts<KT>(en.params, a.params_s, false);
-        accumulate_pair<KT>(en.x1, en.x2, a.out_grad[en.grad_off], kc, acc);
-        owner = (int)en.batch;
+    if (q < a.total) {
+        const Entry en = decode_entry(a, q);
+        if (en.inside) {
+            const KernelConsts kc = make_consts<KT>(en.params, a.params_s, false);
+            accumulate_pair<KT>(en.x1, en.x2, a.out_grad[en.grad_off], kc, acc);
+            owner = (int)en.batch;
+        }
     }
+    // The block's sums (fixed order) and whether all its contributing entries belong to one
+    // batch item: then the second pass takes the sums and never looks at the entries, which are
+    // only written for blocks that mix batch items.
 #pragma unroll
     for (int p = 0; p < KM_MAX_PARAMS; p++) {
-        a.terms[q * KM_MAX_PARAMS + p] = acc[p];
+        sh_sum[p][threadIdx.x] = (double)acc[p];
     }
-    a.owner[q] = owner;
+    sh_lo[threadIdx.x] = owner >= 0 ? owner : 0x7fffffff;
+    sh_hi[threadIdx.x] = owner;
+    __syncthreads();
+    for (int half = 128; half >= 1; half >>= 1) {
+        if ((int)threadIdx.x < half) {
+#pragma unroll
+            for (int p = 0; p < KM_MAX_PARAMS; p++) {
+                sh_sum[p][threadIdx.x] += sh_sum[p][threadIdx.x + half];
+            }
+            sh_lo[threadIdx.x] = min(sh_lo[threadIdx.x], sh_lo[threadIdx.x + half]);
+            sh_hi[threadIdx.x] = max(sh_hi[threadIdx.x], sh_hi[threadIdx.x + half]);
+        }
+        __syncthreads();
+    }
+    const int lo = sh_lo[0], hi = sh_hi[0];
+    if (hi >= 0 && lo != hi && q < a.total) {
+#pragma unroll
+        for (int p = 0; p < KM_MAX_PARAMS; p++) {
+            a.terms[q * KM_MAX_PARAMS + p] = acc[p];
+        }
+        a.owner[q] = owner;
+    }
+    if (threadIdx.x == 0) {
+        a.block_owner[blockIdx.x] = hi < 0 ? -1 : (lo == hi ? lo : -2);
+#pragma unroll
+        for (int p = 0; p < KM_MAX_PARAMS; p++) {
+            a.block_sum[(long long)blockIdx.x * KM_MAX_PARAMS + p] = sh_sum[p][0];
+        }
+    }
 }
 
 template <int KT>
@@ -160,13 +197,58 @@ __global__ void __launch_bounds__(256) index_bwd_reduce(const IndexArgs a) {
     constexpr int P = KernelTraits<KT>::P;
     __shared__ double sh[KM_MAX_PARAMS][256];
     const int b = blockIdx.x;
+    const long long blocks = (a.total + 255) / 256;
+    __shared__ unsigned long long sh_mixed[4][4];  // [quarter][wavefront] which blocks mix batch items
     double sum[KM_MAX_PARAMS] = {0.0, 0.0, 0.0, 0.0};
-    for (long long q = threadIdx.x; q < a.total; q += 256) {
-        if (a.owner[q] == b) {
+    // 1024 blocks at a time, four per thread (their loads in flight together): a block of this
+    // batch item alone adds its sums; blocks that mix batch items are then gone through by the
+    // whole workgroup, one entry per thread.  The order of every thread's additions is fixed.
+    const int wave = threadIdx.x >> 6;
+    for (long long i0 = 0; i0 < blocks; i0 += 1024) {
+        int who[4];
 #pragma unroll
-            for (int p = 0; p < KM_MAX_PARAMS; p++) {
-                sum[p] += (double)a.terms[q * KM_MAX_PARAMS + p];
+        for (int u = 0; u < 4; u++) {
+            const long long i = i0 + 256 * u + threadIdx.x;
+            who[u] = i < blocks ? a.block_owner[i] : -1;
+        }
+        bool mixed = false;
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const long long i = i0 + 256 * u + threadIdx.x;
+            if (who[u] == b) {
+#pragma unroll
+                for (int p = 0; p < KM_MAX_PARAMS; p++) {
+                    sum[p] += a.block_sum[i * KM_MAX_PARAMS + p];
+                }
             }
+            mixed = mixed || who[u] == -2;
+        }
+        if (__syncthreads_or(mixed)) {
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const unsigned long long m = __ballot(who[u] == -2);
+                if ((threadIdx.x & 63) == 0) {
+                    sh_mixed[u][wave] = m;
+                }
+            }
+            __syncthreads();
+            for (int u = 0; u < 4; u++) {
+                for (int w = 0; w < 4; w++) {
+                    unsigned long long m = sh_mixed[u][w];
+                    while (m != 0) {
+                        const int j = __builtin_ctzll(m);
+                        m &= m - 1;
+                        const long long q = (i0 + 256 * u + 64 * w + j) * 256 + threadIdx.x;
+                        if (q < a.total && a.owner[q] == b) {
+#pragma unroll
+                            for (int p = 0; p < KM_MAX_PARAMS; p++) {
+                                sum[p] += (double)a.terms[q * KM_MAX_PARAMS + p];
+                            }
+                        }
+                    }
+                }
+            }
+            __syncthreads();
         }
     }
 #pragma unroll
@@ -255,6 +337,8 @@ static void fill_args(IndexArgs& a, const IndexProblem& p) {
     fill_index(a.out_grad_strides, nullptr, 0);
     a.terms = nullptr;
     a.owner = nullptr;
+    a.block_owner = nullptr;
+    a.block_sum = nullptr;
     a.num_batches = 0;
     a.grad = nullptr;
 }
@@ -280,8 +364,16 @@ hipError_t launch_index(const IndexProblem& p, hipStream_t stream) {
     return hipGetLastError();
 }
 
+// Per entry: KM_MAX_PARAMS terms and the owner; per block of 256 entries: owner and sums.
+static size_t index_bwd_entry_bytes(long long total_entries) {
+    const size_t bytes = (size_t)total_entries * (KM_MAX_PARAMS * sizeof(float) + sizeof(int));
+    return (bytes + 7) & ~(size_t)7;
+}
+
 size_t index_bwd_workspace_bytes(long long total_entries) {
-    return (size_t)total_entries * (KM_MAX_PARAMS * sizeof(float) + sizeof(int));
+    const size_t blocks = (size_t)((total_entries + 255) / 256);
+    return index_bwd_entry_bytes(total_entries) + blocks * KM_MAX_PARAMS * sizeof(double) +
+           blocks * sizeof(int);
 }
 
 hipError_t launch_index_bwd(const IndexBwdProblem& p, hipStream_t stream) {
@@ -291,6 +383,8 @@ hipError_t launch_index_bwd(const IndexBwdProblem& p, hipStream_t stream) {
     fill_index(a.out_grad_strides, p.out_grad_strides, p.index.index_rank);
     a.terms = (float*)p.workspace;
     a.owner = (int*)((char*)p.workspace + (size_t)a.total * KM_MAX_PARAMS * sizeof(float));
+    a.block_sum = (double*)((char*)p.workspace + index_bwd_entry_bytes(a.total));
+    a.block_owner = (int*)(a.block_sum + (size_t)((a.total + 255) / 256) * KM_MAX_PARAMS);
     a.num_batches = p.num_batches;
     a.grad = p.grad;
     const int kt = p.index.kernel_type;

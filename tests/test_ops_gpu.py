@@ -585,3 +585,41 @@ def test_param_grad_coordinate_regimes(regime, kernel_type, vector_width):
     expected = oracle.param_grad(kernel_type, *(f(t) for t in args))
     err = np.abs(result.cpu().double().numpy() - expected)
     assert np.all(err <= _grad_tolerance(expected)), (result.cpu().numpy(), expected)
+
+
+@pytest.mark.parametrize("kernel_type", ["rbf", "spectral", "locally_periodic"])
+def test_index_bwd_blocks_of_one_and_of_several_batch_items(kernel_type):
+    """The diagonal of a batch of matrices as index entries (batch-major, 700 entries per item):
+    blocks of 256 entries that lie inside one batch item go through their block sums, the blocks
+    across an item boundary entry by entry; a second call with the items interleaved entry by
+    entry has no uniform block at all.  Both against the float64 oracle."""
+    from kernel_matmul_amd.configurations import IndexBwdConfiguration
+    from kernel_matmul_amd.ranges import make_ranges
+    from tests.conftest import make_params
+
+    device = torch.device("cuda:0")
+    nb, n = 3, 700
+    x = torch.sort(torch.rand(n) * 10)[0]
+    params = make_params(kernel_type, (nb,))
+    start, end = make_ranges(2.0, x)
+    grads = oracle.kernel_matrix_grad(kernel_type, x.numpy(), x.numpy(), params.numpy())  # [nb, P, n, n]
+    mask = oracle.range_mask(start.numpy(), end.numpy(), n, n)
+    xb, sb, eb = x.to(device).expand(nb, n), start.to(device).expand(nb, -1), end.to(device).expand(nb, -1)
+    for interleaved in (False, True):
+        if interleaved:
+            bi = (torch.arange(nb * n, dtype=torch.int32) % nb).reshape(n, nb)
+            ri = (torch.arange(nb * n, dtype=torch.int32) // nb).reshape(n, nb)
+        else:
+            bi = torch.arange(nb, dtype=torch.int32)[:, None].expand(nb, n).contiguous()
+            ri = torch.arange(n, dtype=torch.int32)[None, :].expand(nb, n).contiguous()
+        ci = torch.clamp(ri + 3, max=n - 1)
+        og = torch.randn(bi.shape)
+        args = (xb, xb, params.to(device), sb, eb, (bi.to(device),), ri.to(device), ci.to(device), og.to(device))
+        result = load_native("index_bwd", IndexBwdConfiguration(kernel_type).make_config(args)).call(*args)
+        expected = np.zeros(params.shape, dtype=np.float64)
+        b_, r_, c_, g_ = (t.numpy().ravel() for t in (bi, ri, ci, og.double()))
+        for q in range(b_.size):
+            if mask[r_[q], c_[q]]:
+                expected[b_[q]] += g_[q] * grads[b_[q], :, r_[q], c_[q]]
+        err = np.abs(result.cpu().double().numpy() - expected)
+        assert np.all(err <= _grad_tolerance(expected) + 1e-6), (interleaved, result.cpu().numpy(), expected)
