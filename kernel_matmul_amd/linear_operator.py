@@ -95,6 +95,8 @@ except ImportError:
             return self._expand_batch(Size(sizes[:-2]))
 
         def diagonal(self) -> Tensor:
+            if hasattr(self, "_diagonal"):
+                return self._diagonal()
             n = min(self.shape[-2], self.shape[-1])
             index = torch.arange(n, device=self.device)
             batch = torch.meshgrid(
@@ -236,6 +238,8 @@ class KernelMatmulLinearOperator(LinearOperator):
         self._batch_shape = batch_shape
         self._symmetric = symmetric
         self._ranges_t = None  # pattern of the transpose, built on first use
+        self._diagonal_indices = None  # index tensors of the diagonal, built on first use
+        self._native_args = None  # (batch shape, widened constructor tensors) of the last call
 
         self._native_matmul = NativeFunction(
             "matmul", MatmulAutotuneConfiguration(kernel_type), compile_pool=compile_pool
@@ -251,16 +255,24 @@ class KernelMatmulLinearOperator(LinearOperator):
 
     # -- helpers -------------------------------------------------------------------------
     def _get_args_for_native(self, batch_shape) -> tuple[Tensor, Tensor, Tensor, Tensor, Tensor]:
+        """The constructor tensors as stride-0 views of ``batch_shape`` (kept for the last shape
+        asked for: solvers call with the same one over and over)."""
+        batch_shape = tuple(batch_shape)
+        if self._native_args is not None and self._native_args[0] == batch_shape:
+            return self._native_args[1]
+
         def widen(t: Tensor, trailing: int) -> Tensor:
             return t.expand(*batch_shape, *t.shape[-trailing:])
 
-        return (
+        args = (
             widen(self._x1.squeeze(-1), 1),
             widen(self._x2.squeeze(-1), 1),
             widen(self._params, 1),
             widen(self._start, 1),
             widen(self._end, 1),
         )
+        self._native_args = (batch_shape, args)
+        return args
 
     def _transposed_ranges(self, batch_shape=None) -> tuple[Tensor, Tensor]:
         """Pattern of K^T, computed once per operator (the check that the pattern is block
@@ -278,10 +290,13 @@ class KernelMatmulLinearOperator(LinearOperator):
 
     # -- LinearOperator hooks ------------------------------------------------------------
     def _matmul(self, rhs: Tensor) -> Tensor:
-        expected = Size((*self._batch_shape, self._x2.size(-2), rhs.size(-1)))
-        broadcast = torch.broadcast_shapes(expected, rhs.shape)
-        batch_shape = broadcast[:-2]
-        rhs_ = rhs.expand(*broadcast)
+        if rhs.shape[:-2] == self._batch_shape and rhs.size(-2) == self._x2.size(-2):
+            batch_shape, rhs_ = self._batch_shape, rhs  # nothing to broadcast
+        else:
+            expected = Size((*self._batch_shape, self._x2.size(-2), rhs.size(-1)))
+            broadcast = torch.broadcast_shapes(expected, rhs.shape)
+            batch_shape = broadcast[:-2]
+            rhs_ = rhs.expand(*broadcast)
         x1, x2, params, start, end = self._get_args_for_native(batch_shape)
         result = _MatmulOperator.apply(
             x1, x2, rhs_, params, start, end, self._native_matmul, self._native_matmul_bwd,
@@ -340,6 +355,27 @@ class KernelMatmulLinearOperator(LinearOperator):
         grad = result.reshape(*batch_shape, result.shape[-1])
         # one entry per constructor tensor: x1, x2, params, start, end
         return None, None, grad, None, None
+
+    def _diagonal(self) -> Tensor:
+        """The diagonal through the index operator, with its index tensors (int32 views that
+        repeat one arange per dimension, no copies) built once per operator instead of by the
+        base class's ``arange`` / ``meshgrid`` / dtype conversion on every call."""
+        if self._diagonal_indices is None:
+            n = min(self._x1.shape[-2], self._x2.shape[-2])
+            batch_shape = tuple(self._batch_shape)
+            device = self._x1.device
+            row = torch.arange(n, dtype=torch.int32, device=device).expand(*batch_shape, n)
+            batch = []
+            for d, size in enumerate(batch_shape):
+                view = [1] * (len(batch_shape) + 1)
+                view[d] = size
+                batch.append(torch.arange(size, dtype=torch.int32, device=device).view(view).expand(*batch_shape, n))
+            self._diagonal_indices = (row, tuple(batch))
+        row, batch = self._diagonal_indices
+        x1, x2, params, start, end = self._get_args_for_native(self._batch_shape)
+        return _IndexOperator.apply(
+            x1, x2, params, start, end, self._native_index, self._native_index_bwd, row, row, *batch
+        )
 
     def _get_indices(self, row_index: Tensor, col_index: Tensor, *batch_indices: Tensor) -> Tensor:
         x1, x2, params, start, end = self._get_args_for_native(self._batch_shape)

@@ -42,6 +42,21 @@ def test_shape_broadcast_and_dtype_device_refusal():
     assert wider.shape == torch.Size((2, 4, 300, 300))
 
 
+def test_widened_constructor_tensors_are_views_kept_for_the_last_batch_shape():
+    x = torch.sort(torch.rand(300, 1), dim=0)[0]
+    params = torch.ones(4, 2)
+    start, end = make_ranges(1.0, x.squeeze(-1))
+    op = KernelMatmulLinearOperator(x, x, params, start, end, kernel_type="rbf")
+    first = op._get_args_for_native(torch.Size((4,)))
+    assert op._get_args_for_native((4,)) is first
+    assert all(t.untyped_storage().data_ptr() == s.untyped_storage().data_ptr()
+               for t, s in zip(first, (x, x, params, start, end)))
+    wider = op._get_args_for_native((2, 4))
+    assert wider is not first and wider[2].shape == (2, 4, 2) and wider[2].stride(0) == 0
+    again = op._get_args_for_native((4,))
+    assert [t.shape for t in again] == [t.shape for t in first]
+
+
 def _make_operator(kernel_type, batch, m, n, device, square, requires_grad=False):
     g = torch.Generator().manual_seed(17)
     x1 = torch.sort(torch.rand(m, generator=g) * 10)[0]
@@ -112,6 +127,25 @@ def test_autograd_params_and_rhs(kernel_type, square):
     dense = _dense(kernel_type, a, batch)
     expected_rhs = np.swapaxes(dense, -1, -2) @ weight.cpu().double().numpy()
     np.testing.assert_allclose(rhs.grad.cpu().numpy(), expected_rhs, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.gpu
+def test_matmul_rhs_batch_shapes_in_turn():
+    """rhs with the operator's batch shape (no broadcast needed), with none, with a wider one,
+    and the first again: each call widens the constructor tensors for its own shape."""
+    device = torch.device("cuda:0")
+    op, _, a = _make_operator("spectral", (3,), 400, 400, device, True)
+    dense = _dense("spectral", a, (3,))
+    g = torch.Generator().manual_seed(5)
+    for shape in [(3, 400, 4), (400, 4), (2, 3, 400, 4), (1, 400, 4), (3, 400, 4)]:
+        rhs = torch.randn(*shape, generator=g)
+        out = op._matmul(rhs.to(device))
+        expected = dense @ rhs.double().numpy()
+        assert out.shape == expected.shape
+        np.testing.assert_allclose(out.cpu().numpy(), expected, rtol=1e-4, atol=1e-5)
+    diag = op.diagonal()
+    np.testing.assert_allclose(diag.cpu().numpy(), np.diagonal(dense, axis1=-2, axis2=-1), rtol=1e-5)
+    np.testing.assert_allclose(op.diagonal().cpu().numpy(), diag.cpu().numpy(), rtol=0)
 
 
 @pytest.mark.gpu
