@@ -316,7 +316,7 @@ def describe_param_grad(kernel_type: str, num_batches: int, m: int, c: int) -> s
     text = ctypes.create_string_buffer(512)
     status = lib.km_param_grad_describe(_kernel_id(kernel_type), num_batches, m, c, text, len(text))
     if status != 0:
-        _raise(status, lib)
+        _raise(lib, status)
     return text.value.decode()
 
 
