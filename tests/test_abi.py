@@ -103,3 +103,8 @@ def test_launch_descriptions_without_a_gpu():
     buf = ctypes.create_string_buffer(16)
     assert lib.km_param_grad_describe(7, 1, 128, 4, buf, len(buf)) == -2
     assert lib.km_param_grad_describe(1, 1, 128, 4, None, 0) == -1
+    # a failed status reaches Python as RuntimeError with the library's message
+    with pytest.raises(RuntimeError, match="km_param_grad_describe: invalid argument"):
+        _native.describe_param_grad("spectral", 1, -5, 4)
+    with pytest.raises(RuntimeError, match="km_matmul_describe: invalid argument"):
+        _native.describe_matmul("spectral", 1, -5, 10, 4)
