@@ -19,6 +19,7 @@ struct DenseArgs {
     long long items_per_xcd;
     int m, n;
     int col_splits;
+    int cols_per_split;    // dense: columns per share, a multiple of 64
     const float* x1;
     const float* x2;
     const float* params;
@@ -59,38 +60,51 @@ __device__ __forceinline__ DenseView dense_view(const DenseArgs& a, long long it
     return v;
 }
 
-// One workgroup of 256 threads per (row block, batch item): each wavefront writes 32 of the
-// block's rows, lanes run along the columns so that stores are 256 B contiguous.
+// One workgroup of 256 threads per (row block, column share, batch item): each wavefront writes
+// 32 of the block's rows over the share's columns, lanes run along the columns so that stores are
+// 256 B contiguous.  The column shares only exist to fill the device when row blocks x batch
+// items are few.  A wavefront keeps its 32 row coordinates one per lane and broadcasts them with
+// v_readlane (no load inside the row loop).
 template <int KT>
 __global__ void __launch_bounds__(256) dense_kernel(const DenseArgs a) {
     const long long item = xcd_item(blockIdx.x, a.items_per_xcd);
     if (item >= a.total_items) {
         return;
     }
-    int row_block, unused;
-    const DenseView v = dense_view(a, item, 1, &row_block, &unused);
-    const KernelConsts kc = make_consts<KT>(v.params, a.params_s, true);
+    int row_block, split;
+    const DenseView v = dense_view(a, item, a.col_splits, &row_block, &split);
+    const int col_lo = split * a.cols_per_split;
+    const int col_hi = min(a.n, col_lo + a.cols_per_split);
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    float* __restrict__ out = a.out + v.b * (long long)a.m * a.n;
     const int row_begin = row_block * KM_BLOCK_SIZE + wave * 32;
-    const int row_end = min(row_begin + 32, a.m);
-    for (int col0 = 0; col0 < a.n; col0 += 64) {
+    const int rows = min(32, a.m - row_begin);
+    if (rows <= 0 || col_lo >= col_hi) {
+        return;
+    }
+    const KernelConsts kc = make_consts<KT>(v.params, a.params_s, true);
+    float* __restrict__ out = a.out + v.b * (long long)a.m * a.n + (long long)row_begin * a.n;
+    const int x1_bits = __float_as_int(v.x1[(long long)(row_begin + min(lane, rows - 1)) * a.x1_s]);
+    for (int col0 = col_lo; col0 < col_hi; col0 += 64) {
         const int col = col0 + lane;
-        const bool in_matrix = col < a.n;
+        const bool in_matrix = col < col_hi;
         const bool in_range = in_matrix && col >= v.range_start && col < v.range_end;
-        // Wave-uniform skip of the evaluation for column tiles fully outside the range.
-        const bool any_in_range = col0 < v.range_end && col0 + 64 > v.range_start;
-        const float x2v = in_range ? v.x2[(long long)col * a.x2_s] : 0.0f;
-        for (int row = row_begin; row < row_end; row++) {
-            float value = 0.0f;
-            if (any_in_range) {
-                const float x1v = v.x1[(long long)row * a.x1_s];
+        float* __restrict__ o = out + col;
+        // Wave-uniform choice: column tiles fully outside the range are only cleared.
+        if (col0 < v.range_end && col0 + 64 > v.range_start) {
+            const float x2v = in_range ? v.x2[(long long)col * a.x2_s] : 0.0f;
+#pragma unroll 4
+            for (int r = 0; r < rows; r++) {
+                const float x1v = __int_as_float(__builtin_amdgcn_readlane(x1_bits, r));
                 const float kv = kernel_value<KT>(x1v, x2v, kc) * kc.sgn;
-                value = in_range ? kv : 0.0f;
+                if (in_matrix) {
+                    o[(long long)r * a.n] = in_range ? kv : 0.0f;
+                }
             }
-            if (in_matrix) {
-                out[(long long)row * a.n + col] = value;
+        } else if (in_matrix) {
+#pragma unroll 4
+            for (int r = 0; r < rows; r++) {
+                o[(long long)r * a.n] = 0.0f;
             }
         }
     }
@@ -116,6 +130,11 @@ __global__ void __launch_bounds__(64) dense_bwd_partial(const DenseArgs a) {
     const int row_begin = row_block * KM_BLOCK_SIZE;
     const int row_end = min(row_begin + KM_BLOCK_SIZE, a.m);
 
+    // The block's 128 row coordinates, two per lane (rows past the matrix repeat the last one;
+    // their weights are zero).
+    const int x1_lo = __float_as_int(v.x1[(long long)min(row_begin + lane, a.m - 1) * a.x1_s]);
+    const int x1_hi = __float_as_int(v.x1[(long long)min(row_begin + 64 + lane, a.m - 1) * a.x1_s]);
+
     float acc[KM_MAX_PARAMS] = {0.0f, 0.0f, 0.0f, 0.0f};
     for (int col0 = col_begin; col0 < col_end; col0 += 64) {
         const int col = col0 + lane;
@@ -123,10 +142,22 @@ __global__ void __launch_bounds__(64) dense_bwd_partial(const DenseArgs a) {
         const int colc = min(col, col_end - 1);
         const float x2v = v.x2[(long long)colc * a.x2_s];
         const float* __restrict__ wcol = v.weights + (long long)colc * a.weights_s1;
-        for (int row = row_begin; row < row_end; row++) {
-            const float x1v = v.x1[(long long)row * a.x1_s];
-            const float wv = ok ? wcol[(long long)row * a.weights_s0] : 0.0f;
-            accumulate_pair<KT>(x1v, x2v, wv, kc, acc);
+        // 8 rows at a time: their weights are requested together, their coordinates come from
+        // the lanes that hold them (below) by v_readlane.
+        for (int row0 = row_begin; row0 < row_end; row0 += 8) {
+            float wv[8];
+#pragma unroll
+            for (int t = 0; t < 8; t++) {
+                const int row = row0 + t;
+                wv[t] = (ok && row < row_end) ? wcol[(long long)row * a.weights_s0] : 0.0f;
+            }
+            const int x1_bits = row0 - row_begin < 64 ? x1_lo : x1_hi;
+            const int first = (row0 - row_begin) & 63;
+#pragma unroll
+            for (int t = 0; t < 8; t++) {
+                const float x1v = __int_as_float(__builtin_amdgcn_readlane(x1_bits, first + t));
+                accumulate_pair<KT>(x1v, x2v, wv[t], kc, acc);
+            }
         }
     }
     const long long partial_rows = a.total_items / a.num_batches;
@@ -170,9 +201,18 @@ hipError_t launch_dense(const DenseProblem& p, hipStream_t stream) {
     collapse_batch<5>(p.batch_rank, p.batch_sizes, strides, &a.batch, outs);
     fill_common(a, p);
     a.weights = nullptr;
-    a.col_splits = 1;
     const long long row_blocks = (p.m + KM_BLOCK_SIZE - 1) / KM_BLOCK_SIZE;
-    a.total_items = row_blocks * p.num_batches;
+    // Column shares of at least 256 columns until there are 2048 workgroups (8 per CU).
+    const long long base = row_blocks * p.num_batches;
+    long long splits = base > 0 ? (2048 + base - 1) / base : 1;
+    const long long most = (p.n + 255) / 256;
+    if (splits > most) splits = most;
+    if (splits < 1) splits = 1;
+    a.cols_per_split = (int)((((p.n + splits - 1) / splits) + 63) / 64 * 64);
+    if (a.cols_per_split < 64) a.cols_per_split = 64;
+    a.col_splits = (int)((p.n + a.cols_per_split - 1) / a.cols_per_split);
+    if (a.col_splits < 1) a.col_splits = 1;
+    a.total_items = row_blocks * a.col_splits * p.num_batches;
     a.items_per_xcd = (a.total_items + KM_NUM_XCD - 1) / KM_NUM_XCD;
     const unsigned grid = (unsigned)(a.items_per_xcd * KM_NUM_XCD);
     switch (p.kernel_type) {
