@@ -178,6 +178,7 @@ __device__ __forceinline__ void pairwise_item(const GradArgs& a, const float* __
 struct GradItem {
     long long b, rest;
     int row0, col_begin, col_end;
+    int width;  // columns of the row block's whole range (all shares)
     const float* x1;
     const float* x2;
     const float* left;
@@ -211,6 +212,7 @@ __device__ __forceinline__ bool grad_item(const GradArgs& a, int rows_per_item, 
     range_end = min(range_end, a.n);
     // Column share of this wavefront, in whole steps of col_step columns.
     const int width = max(range_end - range_start, 0);
+    g->width = width;
     const int per_split = ((width + a.col_splits - 1) / a.col_splits + col_step - 1) & ~(col_step - 1);
     g->col_begin = range_start + split * per_split;
     g->col_end = min(range_end, g->col_begin + per_split);
@@ -247,8 +249,11 @@ __global__ void __launch_bounds__(64) param_grad_partial(const GradArgs a) {
 // The polynomial in h cancels leading terms of size h^2 against a result of size u^2 ~ 1, so the
 // form is only used while |h_i| <= 12 (measured on 1e5 points: the 22-bit products then leave
 // up to 2e-5 of the gradient's largest component, 1e-6 for |h| <= 6), |g_j| <= 48 (dynamic range
-// of the fp16 operands) and every chunk of columns admits the separable exponent; an item that
-// fails any of these is redone in the pairwise form.
+// of the fp16 operands), every chunk of columns admits the separable exponent and the row block's
+// range has at least 64 columns (with a handful of columns nothing averages the rounding of the
+// row sums, measured up to 7e-5 of sum |terms| for a single column against 4e-6 from 64 columns
+// on, and the pairwise form costs next to nothing there); an item that fails any of these is
+// redone in the pairwise form.
 // ---------------------------------------------------------------------------------------
 #define KM_GF_CHUNK 512
 #define KM_GF_MAX_FEATURES 6
@@ -258,6 +263,7 @@ __global__ void __launch_bounds__(64) param_grad_partial(const GradArgs a) {
 #define KM_GF_TABLE_FLOATS (KM_GF_HEAD_FLOATS + KM_BLOCK_SIZE * KM_GF_MAX_WIDTH)
 #define KM_GF_HMAX 12.0f
 #define KM_GF_GMAX 48.0f
+#define KM_GF_MIN_WIDTH 64 /* columns in the row block's range */
 
 template <int KT, int GE, int R, int TL>
 __global__ void __launch_bounds__(64, 2) param_grad_features(const GradArgs a) {
@@ -327,7 +333,8 @@ __global__ void __launch_bounds__(64, 2) param_grad_features(const GradArgs a) {
         row_nan = row_nan || x1v[r] != x1v[r];
     }
     wave_min_max(&row_lo, &row_hi);
-    bool ok = !__any(row_nan) && fmaxf(fabsf(row_hi - c0), fabsf(row_lo - c0)) * kc.s <= KM_GF_HMAX;
+    bool ok = !__any(row_nan) && fmaxf(fabsf(row_hi - c0), fabsf(row_lo - c0)) * kc.s <= KM_GF_HMAX &&
+              g.width >= KM_GF_MIN_WIDTH;
 
     int shift[GE];
     float scale[GE];
