@@ -891,7 +891,7 @@ __global__ void __launch_bounds__(512, 3) fwd_table_f16(const FwdArgs a) {
     // it in scalar registers)
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     fwd_table_f16_body<KT, G, R>(a, lds, w, w.row_block * KM_BLOCK_SIZE + chunk_in_block * (16 * R),
-                                 blockDim.x >> 6, wave, wave, false);
+                                 blockDim.x >> 6, wave, wave, true);
 }
 
 // Grouped launch of the table kernel for large problems (one wavefront per 128-row item, up to
@@ -1015,9 +1015,11 @@ static hipError_t launch_mfma(const FwdArgs& a, int variant, int S, unsigned gx,
     if (variant == KM_VARIANT_MFMA_F16) {
         // The table kernel exists for the shapes the launch table can pick (register budget).
         if constexpr (HAS_TABLE_KERNEL) {
+            // The cross-wavefront reduction buffer lies over the tables (every wavefront is done
+            // with its table by then): less LDS per workgroup, more workgroups per CU.
             const size_t table = (size_t)S * KM_PHASE_TABLE_FLOATS * sizeof(float);
-            hipLaunchKernelGGL((fwd_table_f16<KT, G, R>), dim3(gx, gy, 1), dim3(64 * S, 1, 1), table + lds,
-                               stream, a);
+            hipLaunchKernelGGL((fwd_table_f16<KT, G, R>), dim3(gx, gy, 1), dim3(64 * S, 1, 1),
+                               table > lds ? table : lds, stream, a);
         } else {
             return hipErrorInvalidConfiguration;
         }
