@@ -23,7 +23,7 @@ from typing import List, Tuple
 import torch
 from torch import Size, Tensor, dtype
 
-from kernel_matmul_amd import _BLOCK_SIZE, ranges
+from kernel_matmul_amd import ranges
 from kernel_matmul_amd.configurations import (
     BilinearDerivativeConfiguration,
     DenseBwdConfiguration,
