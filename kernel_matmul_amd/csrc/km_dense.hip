@@ -93,7 +93,6 @@ __global__ void __launch_bounds__(256) dense_kernel(const DenseArgs a) {
         // Wave-uniform choice: column tiles fully outside the range are only cleared.
         if (col0 < v.range_end && col0 + 64 > v.range_start) {
             const float x2v = in_range ? v.x2[(long long)col * a.x2_s] : 0.0f;
-#pragma unroll 4
             for (int r = 0; r < rows; r++) {
                 const float x1v = __int_as_float(__builtin_amdgcn_readlane(x1_bits, r));
                 const float kv = kernel_value<KT>(x1v, x2v, kc) * kc.sgn;
@@ -102,7 +101,6 @@ __global__ void __launch_bounds__(256) dense_kernel(const DenseArgs a) {
                 }
             }
         } else if (in_matrix) {
-#pragma unroll 4
             for (int r = 0; r < rows; r++) {
                 o[(long long)r * a.n] = 0.0f;
             }
