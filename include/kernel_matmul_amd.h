@@ -55,7 +55,9 @@ typedef struct km_launch_options {
     int variant;          /* 0 = table, 1 = VALU FMA contraction, 2 = fp32 MFMA contraction,
                              3 = split-fp16 (hi+lo) MFMA contraction with fp32 accumulation; rbf
                              and spectral kernels with at most 16 rhs columns go through
-                             per-wavefront column tables (spectral in phase-split form),
+                             per-wavefront column tables (spectral in phase-split form), spectral
+                             kernels with 17 to 32 columns too (cosine per entry from tabulated
+                             phases),
                              4 = split-fp16 MFMA with the kernel evaluated directly per pair,
                              5 = split-fp16 MFMA with the rhs operand prepared once per workgroup
                              of four row blocks (rows_per_wave / col_splits must stay 0).

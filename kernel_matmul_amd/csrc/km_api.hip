@@ -134,12 +134,16 @@ static int make_plan(const MatmulProblem& p, const km_launch_options* opt, Matmu
         plan->tail_balance = 0;
         return KM_OK;
     }
-    // Table kernel (column tables in LDS, folded coordinates): rbf and spectral kernels with up
-    // to 16 rhs columns; the spectral one in phase-split form, which keeps two accumulator sets
-    // per rhs column group.  Everything else evaluates directly.
-    const bool table = variant == KM_VARIANT_MFMA_F16 && p.k <= 16 &&
-                       (p.kernel_type == KM_KERNEL_SPECTRAL || p.kernel_type == KM_KERNEL_RBF);
-    const bool phase_split = table && p.kernel_type == KM_KERNEL_SPECTRAL;
+    // Table kernel (column tables in LDS, separable exponent): rbf and spectral kernels with up
+    // to 16 rhs columns, the spectral one in phase-split form (two accumulator sets per rhs
+    // column group); spectral kernels with 17 to 32 columns with the cosine per entry from
+    // tabulated phases (n = 1e5, k = 32, batch 8: 156.6 against 162.8 us direct; n = 1e6: 1.24
+    // against 1.29 ms; the rbf kernel gains nothing from its tables there, 112.9 against 108.7 us).
+    // Everything else evaluates directly.
+    const bool table = variant == KM_VARIANT_MFMA_F16 &&
+                       ((p.k <= 16 && (p.kernel_type == KM_KERNEL_SPECTRAL || p.kernel_type == KM_KERNEL_RBF)) ||
+                        (p.k <= 32 && p.kernel_type == KM_KERNEL_SPECTRAL));
+    const bool phase_split = table && p.kernel_type == KM_KERNEL_SPECTRAL && p.k <= 16;
     if (variant == KM_VARIANT_MFMA_F16 && !table) {
         variant = KM_VARIANT_MFMA_F16_DIRECT;
         plan->variant = variant;
@@ -176,7 +180,7 @@ static int make_plan(const MatmulProblem& p, const km_launch_options* opt, Matmu
     // Kernels at 2 wavefronts per SIMD (the direct kernel at G * R = 16) want 2048 wavefronts
     // before column ranges stop being shared (rbf, n = 65536, k = 64, batch 1: 45.4 us with two
     // wavefronts per row range against 52.9 us with one); the others 1024.
-    const bool two_per_simd = variant == KM_VARIANT_MFMA_F16_DIRECT && G * R >= 16;
+    const bool two_per_simd = (variant == KM_VARIANT_MFMA_F16_DIRECT && G * R >= 16) || (table && G == 2);
     const long long wave_target = two_per_simd ? 2 * TARGET_WAVES : TARGET_WAVES;
     int S = 1;
     if (opt && opt->col_splits != 0) {
@@ -225,13 +229,13 @@ static int make_plan(const MatmulProblem& p, const km_launch_options* opt, Matmu
     // columns.  Measured at n = 1e5, k = 16 (782 items per XCD at batch 8): 12-19 % of an XCD's
     // items split this way is best (112.7 us against 118.7 us with 16-row tail pieces; batch 64:
     // 751 against 773 us); more than a third of a round of wavefronts (128 items) gains nothing.
-    if (table && R == 8 && S == 1 && plan->tail_balance && plan->group_tail < 0) {
+    if (table && G == 1 && R == 8 && S == 1 && plan->tail_balance && plan->group_tail < 0) {
         const long long per_xcd = (row_blocks * p.num_batches + KM_NUM_XCD - 1) / KM_NUM_XCD;
         if (per_xcd >= 2 * 128) {
             plan->group_tail = per_xcd / 7 < 128 ? per_xcd / 7 : 128;
         }
     }
-    if (!(table && R == 8 && S == 1)) {
+    if (!(table && G == 1 && R == 8 && S == 1)) {
         plan->group_tail = -1;
     }
     // The very last of the split items also run as two halves of 64 rows (pieces of an eighth of

@@ -93,6 +93,21 @@ __device__ __forceinline__ void separable_pair_f16(float ra, float rb, float ba,
     *lo = residual_f16x2(ea, one, eb, one, h);
 }
 
+// The same with the oscillating factor of the spectral kernel per entry: times the cosine of
+// the phase difference (revolutions) between the row and each of the two columns.  The low halves
+// are the residuals of the exact products e * cos.
+__device__ __forceinline__ void separable_pair_cos_f16(float ra, float rb, float ba, float bb, float pha,
+                                                       float phb, half2v* hi, half2v* lo) {
+    const float ea = __builtin_amdgcn_exp2f(__builtin_fmaf(ra, ba, rb));
+    const float eb = __builtin_amdgcn_exp2f(__builtin_fmaf(ra, bb, rb));
+    const float ca = __builtin_amdgcn_cosf(pha);
+    const float cb = __builtin_amdgcn_cosf(phb);
+    const float2v kv = {ea * ca, eb * cb};
+    const half2v h = __builtin_convertvector(kv, half2v);
+    *hi = h;
+    *lo = residual_f16x2(ea, ca, eb, cb, h);
+}
+
 __device__ __forceinline__ void split_f16x8(const float (&v)[8], float one, half8v* hi, half8v* lo) {
     half2v h2[4], l2[4];
 #pragma unroll

@@ -6,8 +6,10 @@
 //
 //   fwd_table_f16 : split-fp16 contraction (below) with per-wavefront column tables in LDS
 //                   (x2, scaled x2, and for spectral kernels cos / sin of the column phases:
-//                   phase-split form).  rbf and spectral kernels, up to 16 rhs columns.  The
-//                   kernel the launch table picks for the headline shape.
+//                   phase-split form).  rbf and spectral kernels, up to 16 rhs columns (the
+//                   kernel the launch table picks for the headline shape); spectral kernels
+//                   with 17 to 32 columns keep one accumulator set and take the cosine per
+//                   entry from tabulated column phases.
 //   fwd_mfma_f16  : K entries and rhs are each split into two fp16 terms (hi + lo, 22
 //                   significant bits); the contraction is three v_mfma_f32_16x16x32_f16
 //                   (hi*hi + hi*lo + lo*hi) accumulating in fp32, K evaluated directly per
@@ -331,12 +333,16 @@ __device__ __forceinline__ void f16_load(const FwdArgs& a, const WaveView& w, in
 // which is taken from |rhs| alone.  PARTS = 1 with MULT: every rhs value is multiplied by cb[].
 // SEP: x2v holds b = (x2 - ref) s and the entries are evaluated in the separable form (their
 // column factors 2^(-b^2) come in through cb / sb).
-template <int KT, int G, int R, int KS = KM_F16_KSCALE_LOG2, bool SEP = false, int PARTS = 1, bool MULT = false>
+// PAIRCOS (with SEP): the entries also carry the spectral kernel's cosine, taken per entry from
+// the row phases pa[] and the column phases handed in through sb[] (revolutions).
+template <int KT, int G, int R, int KS = KM_F16_KSCALE_LOG2, bool SEP = false, int PARTS = 1, bool MULT = false,
+          bool PAIRCOS = false>
 __device__ __forceinline__ void f16_step(const float (&x2v)[8], const float (&raw)[G][8],
                                          const float (&x1v)[R], const KernelConsts& kc,
                                          const bool (&colmask)[G], int (&shift)[G],
                                          float (&scale)[G], float4v (&acc)[R][G * PARTS], float ref = 0.0f,
-                                         const float* cb = nullptr, const float* sb = nullptr) {
+                                         const float* cb = nullptr, const float* sb = nullptr,
+                                         const float* pa = nullptr) {
     constexpr int GE = G * PARTS;
     half8v bhi[GE], blo[GE];
 #pragma unroll
@@ -401,7 +407,12 @@ __device__ __forceinline__ void f16_step(const float (&x2v)[8], const float (&ra
             const float rb = __builtin_fmaf(-av, av, (float)KS);
 #pragma unroll
             for (int t = 0; t < 4; t++) {
-                separable_pair_f16(av, rb, x2v[2 * t], x2v[2 * t + 1], kc.one, &h2[t], &l2[t]);
+                if (PAIRCOS) {
+                    separable_pair_cos_f16(av, rb, x2v[2 * t], x2v[2 * t + 1], pa[r] - sb[2 * t],
+                                           pa[r] - sb[2 * t + 1], &h2[t], &l2[t]);
+                } else {
+                    separable_pair_f16(av, rb, x2v[2 * t], x2v[2 * t + 1], kc.one, &h2[t], &l2[t]);
+                }
             }
         } else {
 #pragma unroll
@@ -615,7 +626,12 @@ template <int KT, int G, int R>
 __device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds, const WaveView& wv,
                                                    int row0, int S, int wave, int slot, bool overlay) {
     static_assert(KT == KM_KERNEL_SPECTRAL || KT == KM_KERNEL_RBF, "table kernel: rbf or spectral");
-    constexpr bool PHASE = KT == KM_KERNEL_SPECTRAL;
+    // Spectral kernels: with one group of rhs columns the phase-split form (PHASE: the cosine
+    // leaves the per-entry work for a second accumulator set); with two groups the doubled
+    // accumulators do not fit, and the cosine is taken per entry from tabulated column phases
+    // (PAIRCOS) - still the separable exponent and no phase arithmetic per entry.
+    constexpr bool PHASE = KT == KM_KERNEL_SPECTRAL && G == 1;
+    constexpr bool PAIRCOS = KT == KM_KERNEL_SPECTRAL && G > 1;
     // Accumulator groups; phase-split: [cos part of g = 0..G), sin part of g = 0..G)].
     constexpr int GE = PHASE ? 2 * G : G;
     constexpr int CH = KM_PHASE_CHUNK;
@@ -692,6 +708,13 @@ __device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds,
     wave_min_max(&row_lo, &row_hi);
     const bool rows_finite = !__any(row_nan);
 
+    // Phases of this lane's rows against the reference point (per-entry cosine form only).
+    float row_phase[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        row_phase[r] = PAIRCOS ? phase_rev(kc.f, x1v[r], c_ref) : 0.0f;
+    }
+
     // Tabulates the chunk [chunk0, chunk0 + 512) of this wavefront's columns; returns whether it
     // may take the separable form (then, if `allow`, the column factors already carry 2^(-b^2)).
     auto build = [&](int chunk0, bool allow) -> bool {
@@ -738,6 +761,9 @@ __device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds,
                 tab_sin[q] = __builtin_amdgcn_sinf(th);
             } else {
                 tab_cos[q] = 1.0f;
+                if (PAIRCOS) {
+                    tab_sin[q] = phase_rev(kc.f, xv, c_ref);  // the column's phase itself
+                }
             }
             cols_ok = cols_ok && err == 0.0f && fabsf(b) <= KM_TABLE_SPAN;
             lo = fminf(lo, ref);
@@ -792,7 +818,7 @@ __device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds,
                         cb[t + u] = vc[u];
                     }
                 }
-                if (PHASE) {
+                if (PHASE || (PAIRCOS && SEP)) {
                     const float4v vs = *(const float4v*)(tab_sin + off + t);
 #pragma unroll
                     for (int u = 0; u < 4; u++) {
@@ -801,8 +827,9 @@ __device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds,
                 }
             }
             const float ref = SEP ? tab_ref[off >> 3] : 0.0f;
-            f16_step<KM_KERNEL_RBF, G, R, KS, SEP, GE / G, SEP && !PHASE>(x2v, raw, x1v, kc, colmask, shift,
-                                                                        scale, acc, ref, cb, sb);
+            // (chunks that cannot take the separable form evaluate the whole kernel directly)
+            f16_step<PAIRCOS ? KM_KERNEL_SPECTRAL : KM_KERNEL_RBF, G, R, KS, SEP, GE / G, SEP && !PHASE,
+                     PAIRCOS && SEP>(x2v, raw, x1v, kc, colmask, shift, scale, acc, ref, cb, sb, row_phase);
             if (c0 + 32 < chunk_end) {
                 rhs_load<G>(a, w, c0 + 32, chunk_end, kk, rhs_lane, raw);
             }
@@ -879,7 +906,7 @@ __device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds,
 }
 
 template <int KT, int G, int R>
-__global__ void __launch_bounds__(512, 3) fwd_table_f16(const FwdArgs a) {
+__global__ void __launch_bounds__(512, G == 1 ? 3 : 2) fwd_table_f16(const FwdArgs a) {
     extern __shared__ float lds[];
     const long long item = xcd_item(blockIdx.x, a.items_per_xcd);
     if (item >= a.total_items) {
@@ -1011,7 +1038,8 @@ template <int KT, int G, int R>
 static hipError_t launch_mfma(const FwdArgs& a, int variant, int S, unsigned gx, unsigned gy,
                               hipStream_t stream) {
     const size_t lds = S > 1 ? (size_t)S * R * G * 4 * 64 * sizeof(float) : 0;
-    constexpr bool HAS_TABLE_KERNEL = (KT == KM_KERNEL_SPECTRAL || KT == KM_KERNEL_RBF) && G == 1;
+    constexpr bool HAS_TABLE_KERNEL = ((KT == KM_KERNEL_SPECTRAL || KT == KM_KERNEL_RBF) && G == 1) ||
+                                      (KT == KM_KERNEL_SPECTRAL && G == 2);
     if (variant == KM_VARIANT_MFMA_F16) {
         // The table kernel exists for the shapes the launch table can pick (register budget).
         if constexpr (HAS_TABLE_KERNEL) {

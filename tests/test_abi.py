@@ -91,7 +91,9 @@ def test_launch_descriptions_without_a_gpu():
     """km_matmul_describe / km_param_grad_describe report the launch tables' choices (host only)."""
     text = _native.describe_matmul("spectral", 8, 100_000, 100_000, 16, None)
     assert "fwd_table_f16_grouped<spectral>" in text and "128 rows per wavefront" in text
-    assert "fwd_mfma_f16<spectral" in _native.describe_matmul("spectral", 8, 1_000_000, 1_000_000, 32, None)
+    assert "fwd_table_f16<spectral, G=2" in _native.describe_matmul("spectral", 8, 1_000_000, 1_000_000, 32, None)
+    assert "fwd_mfma_f16<spectral, G=4" in _native.describe_matmul("spectral", 8, 1_000_000, 1_000_000, 64, None)
+    assert "fwd_mfma_f16<rbf, G=2" in _native.describe_matmul("rbf", 8, 1_000_000, 1_000_000, 32, None)
     assert "fwd_table_f16_grouped<rbf>" in _native.describe_matmul("rbf", 8, 1_000_000, 1_000_000, 16, None)
     assert "fwd_block<locally_periodic" in _native.describe_matmul("locally_periodic", 8, 1_000_000, 1_000_000, 16, None)
     # narrow vectors: feature form; wide ones and the locally periodic kernel: pairwise form

@@ -280,16 +280,18 @@ COORDINATE_REGIMES = {
 }
 
 
-@pytest.mark.parametrize("variant", ["auto", "block"])
+@pytest.mark.parametrize("variant,k", [("auto", 16), ("block", 16), ("auto", 24)])
 @pytest.mark.parametrize("kernel_type", ["rbf", "spectral", "locally_periodic"])
 @pytest.mark.parametrize("regime", sorted(COORDINATE_REGIMES))
-def test_matmul_coordinate_regimes(regime, kernel_type, variant):
+def test_matmul_coordinate_regimes(regime, kernel_type, variant, k):
+    """k = 24: two groups of rhs columns (the spectral table kernel then takes the cosine per
+    entry from tabulated column phases instead of the phase-split form)."""
     from kernel_matmul_amd.ranges import make_ranges
     from tests.conftest import make_params
 
     offset, extent, is_sorted = COORDINATE_REGIMES[regime]
     g = torch.Generator().manual_seed(11)
-    m, k, batch = 1500, 16, (2,)
+    m, batch = 1500, (2,)
     x = torch.rand(m, generator=g) * extent + offset
     if is_sorted:
         x = torch.sort(x)[0]
