@@ -563,10 +563,12 @@ __global__ void __launch_bounds__(512) fwd_mfma_f16(const FwdArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------
-// Table kernel (rbf and spectral, up to 16 rhs columns): split-fp16 contraction with
-// per-wavefront column tables in LDS.
+// Table kernel (rbf and spectral up to 16 rhs columns, spectral up to 32): split-fp16
+// contraction with per-wavefront column tables in LDS.
 //
-// Phase-split form (spectral).  With a reference point c per wavefront (its first row) and
+// Phase-split form (spectral, one group of 16 rhs columns; with two groups the second
+// accumulator set does not fit, and the entries carry cos(A_i - B_j) themselves, taken from
+// the row's phase and the tabulated phase of the column).  With a reference point c per wavefront (its first row) and
 // A_i = 2 pi f (x1_i - c), B_j = 2 pi f (x2_j - c):
 //     cos(2 pi f (x1_i - x2_j)) = cos A_i cos B_j + sin A_i sin B_j
 //     out[i,:] = cos A_i * sum_j E_ij (cos B_j rhs[j,:]) + sin A_i * sum_j E_ij (sin B_j rhs[j,:])
