@@ -388,6 +388,37 @@ def test_param_grad_degenerate_ranges(kernel_type):
         assert np.all(err <= _grad_tolerance(expected)), (result.cpu().numpy(), expected)
 
 
+@pytest.mark.parametrize("kernel_type", ["rbf", "spectral"])
+@pytest.mark.parametrize("n", [1, 8, 63])
+def test_bilinear_derivative_narrow_ranges(kernel_type, n):
+    """Ranges of a few columns against a row block that spans many lengthscales: nothing averages
+    the rounding of a row's sums there, so the gradient must come out at the accuracy of a
+    pair-by-pair evaluation, 2e-6 of the sum of |terms| (a form of the gradient that works from
+    moments of the row sums reached 7e-5 on a single column; ranges under 64 columns do not take
+    it)."""
+    g = torch.Generator().manual_seed(31)
+    device = torch.device("cuda:0")
+    m, c = 127, 5
+    for rep in range(4):
+        lengthscale = 0.02
+        x1 = torch.rand(m, generator=g) * 0.4 + 100.0            # unsorted rows, +-8.5 scaled units
+        x2 = torch.sort(torch.rand(n, generator=g) * 0.4 + 100.0)[0]
+        cols = [torch.tensor(lengthscale)] + ([torch.tensor(40.6)] if kernel_type == "spectral" else []) + [torch.tensor(1.1)]
+        params = torch.stack(cols)
+        start = torch.zeros(1, dtype=torch.int32)
+        end = torch.full((1,), n, dtype=torch.int32)
+        left = torch.randn(m, c, generator=g)
+        right = torch.randn(n, c, generator=g)
+        args = tuple(t.to(device) for t in (x1, x2, left, right, params, start, end))
+        defines = BilinearDerivativeConfiguration(kernel_type).make_config(args)
+        result = load_native("bilinear_derivative", defines).call(*args).cpu().double().numpy()
+        f = lambda t: t.numpy()
+        expected = oracle.param_grad(kernel_type, f(x1), f(x2), f(left), f(right), f(params), f(start), f(end))
+        terms = np.abs(oracle.kernel_matrix_grad(kernel_type, f(x1), f(x2), f(params)))
+        size = np.sum(np.abs(left.double().numpy() @ right.double().numpy().T)[None] * terms, axis=(-2, -1))
+        assert np.all(np.abs(result - expected) <= 2e-6 * size + 1e-9), (result, expected, size)
+
+
 def _phase_tolerance(kernel_type, a, rhs64, expected, phase_eps):
     """rtol * |expected| + (atol + phase_eps) * (envelope @ |rhs|): a phase error of phase_eps
     radians changes an entry by that fraction of its envelope (the kernel without its
