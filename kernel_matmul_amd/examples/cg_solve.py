@@ -36,10 +36,14 @@ class ConjugateGradients:
     def __init__(self, kernel_type: str, x: Tensor, params: Tensor, cutoff: float | None, noise: float, k: int):
         self.kernel_type = kernel_type
         batch, n = params.shape[0], x.shape[0]
-        start, end = make_ranges(cutoff, x)
-        self._op_args = (x.expand(batch, n), x.expand(batch, n), params,
-                         start.expand(batch, -1), end.expand(batch, -1))
-        self.noise = noise
+        # Hyper-parameters, pattern and noise live in buffers of their own, so that a captured
+        # iteration keeps reading the current ones after `update`.
+        self.points = x
+        self.params = params.clone()
+        self.range_start, self.range_end = (t.clone() for t in make_ranges(cutoff, x))
+        self.noise = torch.full((1,), float(noise), dtype=torch.float32, device=x.device)
+        self._op_args = (x.expand(batch, n), x.expand(batch, n), self.params,
+                         self.range_start.expand(batch, -1), self.range_end.expand(batch, -1))
         new = lambda *shape: torch.zeros(*shape, dtype=torch.float32, device=x.device)
         self.x = new(batch, n, k)    # iterate
         self.r = new(batch, n, k)    # residual
@@ -57,12 +61,25 @@ class ConjugateGradients:
     def _matvec(self, v: Tensor, out: Tensor) -> None:
         x1, x2, params, start, end = self._op_args
         _native.matmul(self.kernel_type, x1, x2, v, params, start, end, out=out)
-        out.add_(v, alpha=self.noise)
+        out.addcmul_(v, self.noise)
 
     def _column_dots(self, a: Tensor, b: Tensor, out: Tensor) -> None:
         # per-column inner products as a batched (1 x n) @ (n x k) product
         torch.mul(a, b, out=self.tmp)
         torch.bmm(self.ones, self.tmp, out=out)
+
+    def update(self, params: Tensor, cutoff: float | None, noise) -> None:
+        """New hyper-parameters ``(batch, P)``, sparsity cutoff and noise (float or 0-d tensor) for
+        the same points: written into the buffers the iterations read, so a captured graph stays
+        valid."""
+        start, end = make_ranges(cutoff, self.points)
+        self.range_start.copy_(start)
+        self.range_end.copy_(end)
+        self.params.copy_(params)
+        if isinstance(noise, Tensor):
+            self.noise.copy_(noise.reshape(1))
+        else:
+            self.noise.fill_(float(noise))
 
     def start(self, b: Tensor) -> None:
         """x = 0, r = p = b."""
@@ -75,10 +92,12 @@ class ConjugateGradients:
         self._matvec(self.p, self.ap)
         self._column_dots(self.p, self.ap, self.pap)
         torch.div(self.rs, self.pap, out=self.alpha)
+        self.alpha.nan_to_num_(nan=0.0, posinf=0.0, neginf=0.0)  # a column that has converged to 0 / 0
         self.x.addcmul_(self.p, self.alpha)
         self.r.addcmul_(self.ap, self.alpha, value=-1.0)
         self._column_dots(self.r, self.r, self.rs_new)
         torch.div(self.rs_new, self.rs, out=self.beta)
+        self.beta.nan_to_num_(nan=0.0, posinf=0.0, neginf=0.0)
         self.p.mul_(self.beta).add_(self.r)
         self.rs.copy_(self.rs_new)
 

@@ -88,3 +88,22 @@ def test_cg_graph_replays_match_eager_at_full_size():
         rel = float((graphed.rs.sqrt().squeeze(-2) / bd.norm(dim=-2)).max())
         first = rel if first is None else first
     assert rel < 0.5 * first  # the residual goes down
+
+
+def test_update_keeps_a_captured_iteration_valid():
+    """New hyper-parameters, cutoff and noise are written into the buffers the captured iteration
+    reads: replays after `update` equal a solver built from scratch with the new values."""
+    n, batch, k = 4000, 2, 5
+    x, params, b, cutoff = _setup(n, batch, k, seed=73)
+    device = torch.device("cuda:0")
+    xd, bd = x.to(device), b.to(device)
+    graphed = ConjugateGradients("spectral", xd, params.to(device), cutoff, 0.5, k)
+    before = graphed.solve(bd, 8, use_graph=True)[0].clone()   # captures
+    new_params = params * torch.tensor([0.7, 1.3, 1.1])
+    new_cutoff = 6.0 * float(new_params[:, 0].max())
+    graphed.update(new_params.to(device), new_cutoff, torch.tensor(0.3, device=device))
+    fresh = ConjugateGradients("spectral", xd, new_params.to(device), new_cutoff, 0.3, k)
+    sol_g, res_g = graphed.solve(bd, 8, use_graph=True)
+    sol_f, res_f = fresh.solve(bd, 8, use_graph=False)
+    assert torch.equal(sol_g, sol_f) and torch.equal(res_g, res_f)
+    assert not torch.allclose(sol_g, before, rtol=1e-2)
