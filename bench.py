@@ -252,7 +252,7 @@ def main() -> int:
     ap.add_argument("--spin-up-ms", type=float, default=SPIN_UP_MS,
                     help="untimed continuous launches after the warm-up steps (the GPU's clock ramp)")
     ap.add_argument("--workload", default="headline", choices=sorted(WORKLOADS))
-    ap.add_argument("--variant", default="auto", choices=["auto", "block", "mfma_f32", "mfma_f16", "mfma_f16_direct", "valu"])
+    ap.add_argument("--variant", default="auto", choices=["auto", "block", "mfma_f32", "mfma_f32_direct", "mfma_f16", "mfma_f16_direct", "valu"])
     ap.add_argument("--rows-per-wave", type=int, default=0)
     ap.add_argument("--col-splits", type=int, default=0)
     ap.add_argument("--batch", type=int, default=None, help="override the number of batch items")

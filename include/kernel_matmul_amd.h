@@ -52,7 +52,10 @@ extern "C" {
  * (kernel_matmul/configurations.py:84-118): nothing is compiled at run time, the values
  * only select among ahead-of-time instantiated kernels. */
 typedef struct km_launch_options {
-    int variant;          /* 0 = table, 1 = VALU FMA contraction, 2 = fp32 MFMA contraction,
+    int variant;          /* 0 = table, 1 = VALU FMA contraction, 2 = fp32 MFMA contraction (rbf and
+                             spectral kernels with at most 32 rhs columns through the same column
+                             tables as 3, the cosine of the phase difference per entry from
+                             tabulated cosines and sines; others evaluated directly as with 6),
                              3 = split-fp16 (hi+lo) MFMA contraction with fp32 accumulation; rbf
                              and spectral kernels with at most 16 rhs columns go through
                              per-wavefront column tables (spectral in phase-split form), spectral
@@ -60,7 +63,8 @@ typedef struct km_launch_options {
                              phases),
                              4 = split-fp16 MFMA with the kernel evaluated directly per pair,
                              5 = split-fp16 MFMA with the rhs operand prepared once per workgroup
-                             of four row blocks (rows_per_wave / col_splits must stay 0).
+                             of four row blocks (rows_per_wave / col_splits must stay 0),
+                             6 = fp32 MFMA contraction with every entry evaluated directly.
                              The table picks 5 for large locally periodic problems with at most
                              16 rhs columns and 3 otherwise. */
     int rows_per_wave;    /* 0 = table; else 16, 32, 64 or 128 rows of x1 per wavefront */

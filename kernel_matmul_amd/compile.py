@@ -107,7 +107,7 @@ class NativeModule:
         variant = self.defines.get("MATMUL_VARIANT")
         if variant is not None:
             options.variant = {"auto": 0, "valu": 1, "mfma": 2, "mfma_f32": 2, "mfma_f16": 3, "mfma_f16_direct": 4,
-                               "block": 5}[variant]
+                               "block": 5, "mfma_f32_direct": 6}[variant]
         if self.defines.get("MATMUL_TAIL_BALANCE") == 0:
             options.reserved = 1
         elif self.defines.get("MATMUL_GROUP_TAIL") is not None:

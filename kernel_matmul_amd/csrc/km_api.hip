@@ -110,7 +110,7 @@ static int make_plan(const MatmulProblem& p, const km_launch_options* opt, Matmu
         variant = shared ? KM_VARIANT_BLOCK : KM_VARIANT_MFMA_F16;
     }
     if (variant != KM_VARIANT_VALU && variant != KM_VARIANT_MFMA_F32 && variant != KM_VARIANT_MFMA_F16 &&
-        variant != KM_VARIANT_MFMA_F16_DIRECT && variant != KM_VARIANT_BLOCK) {
+        variant != KM_VARIANT_MFMA_F16_DIRECT && variant != KM_VARIANT_BLOCK && variant != KM_VARIANT_MFMA_F32_DIRECT) {
         return fail(KM_ERR_INVALID_ARGUMENT, "km_matmul: unknown variant %d", variant);
     }
     if (variant == KM_VARIANT_BLOCK) {
@@ -140,12 +140,19 @@ static int make_plan(const MatmulProblem& p, const km_launch_options* opt, Matmu
     // tabulated phases (n = 1e5, k = 32, batch 8: 156.6 against 162.8 us direct; n = 1e6: 1.24
     // against 1.29 ms; the rbf kernel gains nothing from its tables there, 112.9 against 108.7 us).
     // Everything else evaluates directly.
-    const bool table = variant == KM_VARIANT_MFMA_F16 &&
-                       ((p.k <= 16 && (p.kernel_type == KM_KERNEL_SPECTRAL || p.kernel_type == KM_KERNEL_RBF)) ||
-                        (p.k <= 32 && p.kernel_type == KM_KERNEL_SPECTRAL));
-    const bool phase_split = table && p.kernel_type == KM_KERNEL_SPECTRAL && p.k <= 16;
+    // The fp32 contraction goes through the same tables for rbf and spectral kernels up to 32
+    // columns (cos(A - B) per entry from tabulated cos B / sin B); otherwise directly as well.
+    const bool rbf_or_spectral = p.kernel_type == KM_KERNEL_SPECTRAL || p.kernel_type == KM_KERNEL_RBF;
+    const bool table = (variant == KM_VARIANT_MFMA_F16 &&
+                        ((p.k <= 16 && rbf_or_spectral) || (p.k <= 32 && p.kernel_type == KM_KERNEL_SPECTRAL))) ||
+                       (variant == KM_VARIANT_MFMA_F32 && p.k <= 32 && rbf_or_spectral);
+    const bool phase_split = variant == KM_VARIANT_MFMA_F16 && table && p.kernel_type == KM_KERNEL_SPECTRAL && p.k <= 16;
     if (variant == KM_VARIANT_MFMA_F16 && !table) {
         variant = KM_VARIANT_MFMA_F16_DIRECT;
+        plan->variant = variant;
+    }
+    if (variant == KM_VARIANT_MFMA_F32 && !table) {
+        variant = KM_VARIANT_MFMA_F32_DIRECT;
         plan->variant = variant;
     }
     plan->k_chunk = p.k <= 16 ? 16 : ((p.k <= 32 || phase_split) ? 32 : 64);
@@ -180,7 +187,8 @@ static int make_plan(const MatmulProblem& p, const km_launch_options* opt, Matmu
     // Kernels at 2 wavefronts per SIMD (the direct kernel at G * R = 16) want 2048 wavefronts
     // before column ranges stop being shared (rbf, n = 65536, k = 64, batch 1: 45.4 us with two
     // wavefronts per row range against 52.9 us with one); the others 1024.
-    const bool two_per_simd = (variant == KM_VARIANT_MFMA_F16_DIRECT && G * R >= 16) || (table && G == 2);
+    const bool two_per_simd = (variant == KM_VARIANT_MFMA_F16_DIRECT && G * R >= 16) ||
+                              (variant == KM_VARIANT_MFMA_F16 && table && G == 2);
     const long long wave_target = two_per_simd ? 2 * TARGET_WAVES : TARGET_WAVES;
     int S = 1;
     if (opt && opt->col_splits != 0) {
@@ -477,15 +485,17 @@ int km_matmul_describe(int kernel_type, int64_t num_batches, int64_t m, int64_t 
                      kt, plan.phase_split, G);
             break;
         default: {
-            const char* name = plan.variant == KM_VARIANT_MFMA_F32
+            const char* name = plan.variant == KM_VARIANT_MFMA_F32_DIRECT
                                    ? "km::fwd_mfma_f32"
-                                   : (plan.variant == KM_VARIANT_MFMA_F16 ? "km::fwd_table_f16" : "km::fwd_mfma_f16");
-            if (plan.variant == KM_VARIANT_MFMA_F16 && plan.group_tail >= 0) {
+                                   : (plan.variant == KM_VARIANT_MFMA_F32
+                                          ? "km::fwd_table_f32"
+                                          : (plan.variant == KM_VARIANT_MFMA_F16 ? "km::fwd_table_f16" : "km::fwd_mfma_f16"));
+            if ((plan.variant == KM_VARIANT_MFMA_F16 || plan.variant == KM_VARIANT_MFMA_F32) && plan.group_tail >= 0) {
                 snprintf(text, text_bytes,
-                         "km::fwd_table_f16_grouped<%s>: 128 rows per wavefront, 4 wavefronts per workgroup, the "
+                         "%s_grouped<%s>: 128 rows per wavefront, 4 wavefronts per workgroup, the "
                          "last %lld items of each XCD split by columns over a workgroup (the last %lld of them "
                          "also into two halves of 64 rows)",
-                         kt, plan.group_tail, plan.group_tail_halves);
+                         name, kt, plan.group_tail, plan.group_tail_halves);
                 break;
             }
             snprintf(text, text_bytes, "%s<%s, G=%d, R=%d>: %d rows per wavefront, %d wavefront(s) per row range%s",

@@ -10,10 +10,11 @@ namespace km {
 enum {
     KM_VARIANT_AUTO = 0,
     KM_VARIANT_VALU = 1,
-    KM_VARIANT_MFMA_F32 = 2,
+    KM_VARIANT_MFMA_F32 = 2,         // fp32 MFMA; rbf and spectral kernels up to 32 rhs columns through the column tables
     KM_VARIANT_MFMA_F16 = 3,         // split-fp16 MFMA; spectral kernels in phase-split form
     KM_VARIANT_MFMA_F16_DIRECT = 4,  // split-fp16 MFMA with the cosine evaluated per pair
-    KM_VARIANT_BLOCK = 5             // split-fp16 MFMA, rhs operand prepared once per workgroup of 4 row blocks
+    KM_VARIANT_BLOCK = 5,            // split-fp16 MFMA, rhs operand prepared once per workgroup of 4 row blocks
+    KM_VARIANT_MFMA_F32_DIRECT = 6   // fp32 MFMA with every entry evaluated directly, operands straight from memory
 };
 
 struct MatmulProblem {

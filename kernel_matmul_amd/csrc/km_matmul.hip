@@ -436,6 +436,61 @@ __device__ __forceinline__ void f16_step(const float (&x2v)[8], const float (&ra
     }
 }
 
+// One step of 32 columns with the contraction in fp32 (v_mfma_f32_16x16x4_f32, 8 per row group and
+// rhs column group): MFMA t of the step contracts the columns {8 kk + t}, so a lane evaluates its
+// row against the same 8 consecutive columns as in the split-fp16 step and the column tables are
+// shared.  Entries (K / sigma):
+//   SEP      2^(a * 2b - a^2), the column factor 2^(-b^2) carried by cb / sb (spectral) or
+//            multiplied into the rhs operand (rbf); x2v holds 2b
+//   else     2^(-((x1 - x2) s)^2); x2v holds x2
+//   spectral times cos(A_i - B_j) = cos A_i cos B_j + sin A_i sin B_j from the row's ca / sa and the
+//            tabulated cb / sb: two full-rate operations instead of a phase product and a cosine.
+template <int KT, int G, int R, bool SEP>
+__device__ __forceinline__ void f32_step(const float (&x2v)[8], const float (&raw)[G][8],
+                                         const float (&x1v)[R], const KernelConsts& kc,
+                                         float4v (&acc)[R][G], float ref, const float (&cb)[8],
+                                         const float (&sb)[8], const float (&ca)[R], const float (&sa)[R]) {
+    float bv[G][8];
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+            bv[g][t] = (SEP && KT == KM_KERNEL_RBF) ? raw[g][t] * cb[t] : raw[g][t];
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        float kv[8];
+        if (SEP) {
+            const float av = (x1v[r] - ref) * kc.s;
+            const float rb = -av * av;
+#pragma unroll
+            for (int t = 0; t < 8; t++) {
+                kv[t] = __builtin_amdgcn_exp2f(__builtin_fmaf(av, x2v[t], rb));
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < 8; t++) {
+                const float u = (x1v[r] - x2v[t]) * kc.s;
+                kv[t] = __builtin_amdgcn_exp2f(-u * u);
+            }
+        }
+        if (KT == KM_KERNEL_SPECTRAL) {
+#pragma unroll
+            for (int t = 0; t < 8; t++) {
+                kv[t] *= __builtin_fmaf(sa[r], sb[t], ca[r] * cb[t]);
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                acc[r][g] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv[t], bv[g][t], acc[r][g], 0, 0, 0);
+            }
+        }
+    }
+}
+
 // PF: request the next step's operands before evaluating the current one (costs 8 + 8 G
 // registers; used for G = 1 where they are available).
 template <int KT, int G, int R, bool PF>
@@ -624,21 +679,25 @@ __device__ __forceinline__ void rhs_load(const FwdArgs& a, const WaveView& w, in
 // S wavefronts (this one is number `wave` of them) share the row range and split its columns;
 // `slot` is the wavefront's table area in LDS.  With `overlay` the cross-wavefront reduction
 // buffer lies over the table areas instead of behind them.
-template <int KT, int G, int R>
-__device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds, const WaveView& wv,
+template <int KT, int G, int R, bool F32 = false>
+__device__ __forceinline__ void fwd_table_body(const FwdArgs& a, float* lds, const WaveView& wv,
                                                    int row0, int S, int wave, int slot, bool overlay) {
     static_assert(KT == KM_KERNEL_SPECTRAL || KT == KM_KERNEL_RBF, "table kernel: rbf or spectral");
     // Spectral kernels: with one group of rhs columns the phase-split form (PHASE: the cosine
     // leaves the per-entry work for a second accumulator set); with two groups the doubled
     // accumulators do not fit, and the cosine is taken per entry from tabulated column phases
     // (PAIRCOS) - still the separable exponent and no phase arithmetic per entry.
-    constexpr bool PHASE = KT == KM_KERNEL_SPECTRAL && G == 1;
-    constexpr bool PAIRCOS = KT == KM_KERNEL_SPECTRAL && G > 1;
+    // F32: the contraction is an fp32 MFMA on the evaluated entries themselves (no split, no
+    // scales); spectral entries take cos(A_i - B_j) from the tabulated cos B / sin B and the row's
+    // cos A / sin A (TRIG).
+    constexpr bool PHASE = !F32 && KT == KM_KERNEL_SPECTRAL && G == 1;
+    constexpr bool PAIRCOS = !F32 && KT == KM_KERNEL_SPECTRAL && G > 1;
+    constexpr bool TRIG = F32 && KT == KM_KERNEL_SPECTRAL;
     // Accumulator groups; phase-split: [cos part of g = 0..G), sin part of g = 0..G)].
     constexpr int GE = PHASE ? 2 * G : G;
     constexpr int CH = KM_PHASE_CHUNK;
     constexpr int PER_LANE = CH / 64;
-    constexpr int KS = KM_TABLE_KSCALE_LOG2;
+    constexpr int KS = F32 ? 0 : KM_TABLE_KSCALE_LOG2;
 
     const int lane = threadIdx.x & 63;
     const int li = lane & 15;
@@ -676,7 +735,7 @@ __device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds,
         const int c = kbase + 16 * g + li;
         rhs_lane[g] = (unsigned)(8 * kk * a.rhs_s0 + (min(c, a.k - 1) - kbase) * a.rhs_s1);
         colmask[g] = c < a.k;
-        shift[g] = 100;
+        shift[g] = F32 ? 0 : 100;
         scale[g] = c < a.k ? __builtin_ldexpf(1.0f, 100) : 0.0f;
     }
 
@@ -715,6 +774,14 @@ __device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds,
 #pragma unroll
     for (int r = 0; r < R; r++) {
         row_phase[r] = PAIRCOS ? phase_rev(kc.f, x1v[r], c_ref) : 0.0f;
+    }
+    // Cosine and sine of the same phases (fp32 contraction: the lane's row of the A operand).
+    float row_cos[R], row_sin[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const float th = TRIG ? phase_rev(kc.f, x1v[r], c_ref) : 0.0f;
+        row_cos[r] = TRIG ? __builtin_amdgcn_cosf(th) : 1.0f;
+        row_sin[r] = TRIG ? __builtin_amdgcn_sinf(th) : 0.0f;
     }
 
     // Tabulates the chunk [chunk0, chunk0 + 512) of this wavefront's columns; returns whether it
@@ -757,7 +824,7 @@ __device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds,
             const float err = (xv - (xd - bb)) - (ref + bb);  // exact rounding error of xd
             const float b = xd * kc.s;
             tab_b[q] = b;
-            if (PHASE) {
+            if (PHASE || TRIG) {
                 const float th = phase_rev(kc.f, xv, c_ref);
                 tab_cos[q] = __builtin_amdgcn_cosf(th);
                 tab_sin[q] = __builtin_amdgcn_sinf(th);
@@ -785,7 +852,7 @@ __device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds,
                 const float wgt = __builtin_amdgcn_exp2f(-b * b);
                 tab_b[q] = b + b;
                 tab_cos[q] *= wgt;
-                if (PHASE) {
+                if (PHASE || TRIG) {
                     tab_sin[q] *= wgt;
                 }
             }
@@ -813,14 +880,14 @@ __device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds,
                 for (int u = 0; u < 4; u++) {
                     x2v[t + u] = vx[u];
                 }
-                if (PHASE || SEP) {
+                if (PHASE || TRIG || SEP) {
                     const float4v vc = *(const float4v*)(tab_cos + off + t);
 #pragma unroll
                     for (int u = 0; u < 4; u++) {
                         cb[t + u] = vc[u];
                     }
                 }
-                if (PHASE || (PAIRCOS && SEP)) {
+                if (PHASE || TRIG || (PAIRCOS && SEP)) {
                     const float4v vs = *(const float4v*)(tab_sin + off + t);
 #pragma unroll
                     for (int u = 0; u < 4; u++) {
@@ -830,8 +897,12 @@ __device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds,
             }
             const float ref = SEP ? tab_ref[off >> 3] : 0.0f;
             // (chunks that cannot take the separable form evaluate the whole kernel directly)
-            f16_step<PAIRCOS ? KM_KERNEL_SPECTRAL : KM_KERNEL_RBF, G, R, KS, SEP, GE / G, SEP && !PHASE,
-                     PAIRCOS && SEP>(x2v, raw, x1v, kc, colmask, shift, scale, acc, ref, cb, sb, row_phase);
+            if constexpr (F32) {
+                f32_step<KT, G, R, SEP>(x2v, raw, x1v, kc, acc, ref, cb, sb, row_cos, row_sin);
+            } else {
+                f16_step<PAIRCOS ? KM_KERNEL_SPECTRAL : KM_KERNEL_RBF, G, R, KS, SEP, GE / G, SEP && !PHASE,
+                         PAIRCOS && SEP>(x2v, raw, x1v, kc, colmask, shift, scale, acc, ref, cb, sb, row_phase);
+            }
             if (c0 + 32 < chunk_end) {
                 rhs_load<G>(a, w, c0 + 32, chunk_end, kk, rhs_lane, raw);
             }
@@ -907,9 +978,8 @@ __device__ __forceinline__ void fwd_table_f16_body(const FwdArgs& a, float* lds,
     }
 }
 
-template <int KT, int G, int R>
-__global__ void __launch_bounds__(512, G == 1 ? 3 : 2) fwd_table_f16(const FwdArgs a) {
-    extern __shared__ float lds[];
+template <int KT, int G, int R, bool F32>
+__device__ __forceinline__ void fwd_table_kernel(const FwdArgs& a, float* lds) {
     const long long item = xcd_item(blockIdx.x, a.items_per_xcd);
     if (item >= a.total_items) {
         return;
@@ -919,8 +989,21 @@ __global__ void __launch_bounds__(512, G == 1 ? 3 : 2) fwd_table_f16(const FwdAr
     // (the wavefront index is wave-uniform by construction; saying so keeps what is derived from
     // it in scalar registers)
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    fwd_table_f16_body<KT, G, R>(a, lds, w, w.row_block * KM_BLOCK_SIZE + chunk_in_block * (16 * R),
-                                 blockDim.x >> 6, wave, wave, true);
+    fwd_table_body<KT, G, R, F32>(a, lds, w, w.row_block * KM_BLOCK_SIZE + chunk_in_block * (16 * R),
+                                  blockDim.x >> 6, wave, wave, true);
+}
+
+template <int KT, int G, int R>
+__global__ void __launch_bounds__(512, G == 1 ? 3 : 2) fwd_table_f16(const FwdArgs a) {
+    extern __shared__ float lds[];
+    fwd_table_kernel<KT, G, R, false>(a, lds);
+}
+
+// The same with the contraction as fp32 MFMAs (f32_step).
+template <int KT, int G, int R>
+__global__ void __launch_bounds__(512, G == 1 ? 3 : 2) fwd_table_f32(const FwdArgs a) {
+    extern __shared__ float lds[];
+    fwd_table_kernel<KT, G, R, true>(a, lds);
 }
 
 // Grouped launch of the table kernel for large problems (one wavefront per 128-row item, up to
@@ -931,9 +1014,8 @@ __global__ void __launch_bounds__(512, G == 1 ? 3 : 2) fwd_table_f16(const FwdAr
 // while the last full items finish.
 #define KM_GROUP_WAVES 4
 
-template <int KT>
-__global__ void __launch_bounds__(64 * KM_GROUP_WAVES, 3) fwd_table_f16_grouped(const FwdArgs a) {
-    extern __shared__ float lds[];
+template <int KT, bool F32>
+__device__ __forceinline__ void fwd_table_grouped_kernel(const FwdArgs& a, float* lds) {
     // The wavefront index is wave-uniform by construction; saying so keeps the item and
     // everything derived from it (pointers, ranges, parameters) in scalar registers.
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -965,12 +1047,24 @@ __global__ void __launch_bounds__(64 * KM_GROUP_WAVES, 3) fwd_table_f16_grouped(
     int unused;
     const WaveView w = wave_view(a, item, 1, &unused);
     if (halves) {
-        fwd_table_f16_body<KT, 1, 4>(a, lds, w, w.row_block * KM_BLOCK_SIZE + 64 * half, KM_GROUP_WAVES, wave, wave,
-                                     true);
+        fwd_table_body<KT, 1, 4, F32>(a, lds, w, w.row_block * KM_BLOCK_SIZE + 64 * half, KM_GROUP_WAVES, wave, wave,
+                                      true);
     } else {
-        fwd_table_f16_body<KT, 1, 8>(a, lds, w, w.row_block * KM_BLOCK_SIZE, split ? KM_GROUP_WAVES : 1,
-                                     split ? wave : 0, wave, true);
+        fwd_table_body<KT, 1, 8, F32>(a, lds, w, w.row_block * KM_BLOCK_SIZE, split ? KM_GROUP_WAVES : 1,
+                                      split ? wave : 0, wave, true);
     }
+}
+
+template <int KT>
+__global__ void __launch_bounds__(64 * KM_GROUP_WAVES, 3) fwd_table_f16_grouped(const FwdArgs a) {
+    extern __shared__ float lds[];
+    fwd_table_grouped_kernel<KT, false>(a, lds);
+}
+
+template <int KT>
+__global__ void __launch_bounds__(64 * KM_GROUP_WAVES, 3) fwd_table_f32_grouped(const FwdArgs a) {
+    extern __shared__ float lds[];
+    fwd_table_grouped_kernel<KT, true>(a, lds);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -1058,6 +1152,14 @@ static hipError_t launch_mfma(const FwdArgs& a, int variant, int S, unsigned gx,
         // picks them.
         if constexpr (G * R <= 16) {
             hipLaunchKernelGGL((fwd_mfma_f16<KT, G, R, G == 1>), dim3(gx, gy, 1), dim3(64 * S, 1, 1), lds, stream, a);
+        } else {
+            return hipErrorInvalidConfiguration;
+        }
+    } else if (variant == KM_VARIANT_MFMA_F32) {
+        if constexpr ((KT == KM_KERNEL_SPECTRAL || KT == KM_KERNEL_RBF) && G <= 2) {
+            const size_t table = (size_t)S * KM_PHASE_TABLE_FLOATS * sizeof(float);
+            hipLaunchKernelGGL((fwd_table_f32<KT, G, R>), dim3(gx, gy, 1), dim3(64 * S, 1, 1),
+                               table > lds ? table : lds, stream, a);
         } else {
             return hipErrorInvalidConfiguration;
         }
@@ -1168,8 +1270,9 @@ hipError_t launch_matmul(const MatmulProblem& p, const MatmulPlan& plan, hipStre
             default: return launch_valu<KM_KERNEL_LOCALLY_PERIODIC>(a, plan.k_chunk, grid_x, grid_y, stream);
         }
     }
-    if (plan.variant == KM_VARIANT_MFMA_F16 && plan.group_tail >= 0 && plan.row_groups == 8 &&
-        plan.col_splits == 1 && plan.k_chunk == 16 && p.kernel_type != KM_KERNEL_LOCALLY_PERIODIC) {
+    if ((plan.variant == KM_VARIANT_MFMA_F16 || plan.variant == KM_VARIANT_MFMA_F32) && plan.group_tail >= 0 &&
+        plan.row_groups == 8 && plan.col_splits == 1 && plan.k_chunk == 16 &&
+        p.kernel_type != KM_KERNEL_LOCALLY_PERIODIC) {
         a.tail_items = (int)(plan.group_tail < a.items_per_xcd ? plan.group_tail : a.items_per_xcd);
         a.tail_half_items = (int)(plan.group_tail_halves < a.tail_items ? plan.group_tail_halves : a.tail_items);
         const long long main_groups = (a.items_per_xcd - a.tail_items + KM_GROUP_WAVES - 1) / KM_GROUP_WAVES;
@@ -1177,7 +1280,15 @@ hipError_t launch_matmul(const MatmulProblem& p, const MatmulPlan& plan, hipStre
         const size_t table = (size_t)KM_GROUP_WAVES * KM_PHASE_TABLE_FLOATS * sizeof(float);
         static_assert(KM_GROUP_WAVES * 8 * 4 * 64 <= KM_GROUP_WAVES * KM_PHASE_TABLE_FLOATS,
                       "the reduction buffer of a split item must fit over the tables");
-        if (p.kernel_type == KM_KERNEL_SPECTRAL) {
+        if (plan.variant == KM_VARIANT_MFMA_F32) {
+            if (p.kernel_type == KM_KERNEL_SPECTRAL) {
+                hipLaunchKernelGGL((fwd_table_f32_grouped<KM_KERNEL_SPECTRAL>), dim3(gx, grid_y, 1),
+                                   dim3(64 * KM_GROUP_WAVES, 1, 1), table, stream, a);
+            } else {
+                hipLaunchKernelGGL((fwd_table_f32_grouped<KM_KERNEL_RBF>), dim3(gx, grid_y, 1),
+                                   dim3(64 * KM_GROUP_WAVES, 1, 1), table, stream, a);
+            }
+        } else if (p.kernel_type == KM_KERNEL_SPECTRAL) {
             hipLaunchKernelGGL((fwd_table_f16_grouped<KM_KERNEL_SPECTRAL>), dim3(gx, grid_y, 1),
                                dim3(64 * KM_GROUP_WAVES, 1, 1), table, stream, a);
         } else {

@@ -48,6 +48,7 @@ def test_matmul(example_data, col_blocks):
 
 
 @pytest.mark.parametrize("variant,rows", [("valu", None), ("mfma_f32", 16), ("mfma_f32", 32), ("mfma_f32", 64), ("mfma_f32", 128),
+                                          ("mfma_f32_direct", 32), ("mfma_f32_direct", 128),
                                           ("mfma_f16", 16), ("mfma_f16", 32), ("mfma_f16", 64), ("mfma_f16", 128),
                                           ("mfma_f16_direct", 32), ("mfma_f16_direct", 128), ("block", None)])
 def test_matmul_variants(example_data, variant, rows):
@@ -63,7 +64,7 @@ def test_matmul_variants(example_data, variant, rows):
     assert_close(result, expected)
 
 
-@pytest.mark.parametrize("variant", ["auto", "block", "mfma_f16_direct", "mfma_f32"])
+@pytest.mark.parametrize("variant", ["auto", "block", "mfma_f16_direct", "mfma_f32", "mfma_f32_direct"])
 def test_matmul_rhs_dynamic_range(example_data, variant):
     """rhs whose magnitude spans 12 decades across columns and e^24 along the rows: the
     half-precision contraction rescales its operands per column while it walks a row range, so
@@ -98,7 +99,7 @@ def test_matmul_rhs_dynamic_range(example_data, variant):
     else:
         bound = np.abs(kd) @ np.abs(rhs64)
     floor = 0.0
-    if variant != "mfma_f32":
+    if variant not in ("mfma_f32", "mfma_f32_direct"):
         start, end = a["start"].copy(), a["end"].copy()
         if variant == "block":
             for g0 in range(0, start.shape[-1], 4):
@@ -280,7 +281,7 @@ COORDINATE_REGIMES = {
 }
 
 
-@pytest.mark.parametrize("variant,k", [("auto", 16), ("block", 16), ("auto", 24)])
+@pytest.mark.parametrize("variant,k", [("auto", 16), ("block", 16), ("auto", 24), ("mfma_f32", 16), ("mfma_f32", 24)])
 @pytest.mark.parametrize("kernel_type", ["rbf", "spectral", "locally_periodic"])
 @pytest.mark.parametrize("regime", sorted(COORDINATE_REGIMES))
 def test_matmul_coordinate_regimes(regime, kernel_type, variant, k):
@@ -319,7 +320,7 @@ def test_matmul_coordinate_regimes(regime, kernel_type, variant, k):
     assert_close(result, expected)
 
 
-@pytest.mark.parametrize("variant", ["auto", "block", "mfma_f16_direct", "mfma_f32", "valu"])
+@pytest.mark.parametrize("variant", ["auto", "block", "mfma_f16_direct", "mfma_f32", "mfma_f32_direct", "valu"])
 @pytest.mark.parametrize("kernel_type", ["rbf", "spectral"])
 def test_matmul_degenerate_ranges(kernel_type, variant):
     """Row blocks with an empty range must produce exact zeros (the output is fully written),
@@ -432,7 +433,7 @@ def _phase_tolerance(kernel_type, a, rhs64, expected, phase_eps):
     return RTOL * np.abs(expected) + (ATOL + phase_eps) * (np.abs(env) @ np.abs(rhs64)) + 1e-30
 
 
-@pytest.mark.parametrize("variant", ["auto", "block", "mfma_f16_direct", "mfma_f32"])
+@pytest.mark.parametrize("variant", ["auto", "block", "mfma_f16_direct", "mfma_f32", "mfma_f32_direct"])
 @pytest.mark.parametrize("frequency", [5.0, 50.0])
 def test_matmul_spectral_high_frequency(frequency, variant):
     """Spectral kernels with many oscillations per window (up to 125 revolutions across the
@@ -494,7 +495,7 @@ def _far_phase_problem(kernel_type, k):
 
 @pytest.mark.parametrize("kernel_type", ["spectral", "locally_periodic"])
 @pytest.mark.parametrize("variant,k", [("auto", 16), ("auto", 32), ("block", 16), ("mfma_f16_direct", 32),
-                                       ("mfma_f32", 16), ("valu", 8)])
+                                       ("mfma_f32", 16), ("mfma_f32", 32), ("mfma_f32_direct", 16), ("valu", 8)])
 def test_matmul_phase_beyond_256_revolutions(kernel_type, variant, k):
     t, a, phase_eps = _far_phase_problem(kernel_type, k)
     args = (t["x"], t["x"], t["rhs"], t["params"], t["start"], t["end"])

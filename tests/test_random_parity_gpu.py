@@ -63,7 +63,7 @@ def _draw(rng):
         width = torch.randint(0, n + 1, (*batch, rows), dtype=torch.int32)
         end = torch.minimum(start + width, torch.tensor(n, dtype=torch.int32))
     rhs = torch.randn(*batch, n, k) * rng.choice([1.0, 1e-3, 1e3])
-    variant = rng.choice([None, None, None, "mfma_f16", "mfma_f16_direct", "block", "mfma_f32", "valu"])
+    variant = rng.choice([None, None, None, "mfma_f16", "mfma_f16_direct", "block", "mfma_f32", "mfma_f32_direct", "valu"])
     rows_per_wave = rng.choice([None, None, 16, 32, 64, 128])
     splits = rng.choice([None, None, 1, 2, 4, 8])
     c = rng.choice([1, 3, 4, 5, 8, 10, 16])
