@@ -864,12 +864,22 @@ __device__ __forceinline__ void fwd_table_body(const FwdArgs& a, float* lds, con
         return separable;
     };
 
+    // rhs operand of the current step.  The fp32 kernel (registers to spare) requests a chunk's
+    // first step before the chunk is tabulated, so the two memory round trips overlap.
+    float raw[G][8];
+    auto request_first = [&](int chunk0) {
+        if (F32) {
+            rhs_load<G>(a, w, chunk0, min(chunk0 + CH, col_end), kk, rhs_lane, raw);
+        }
+    };
+
     // The steps of a tabulated chunk.
     auto steps = [&](int chunk0, auto sep_c) {
         constexpr bool SEP = decltype(sep_c)::value;
         const int chunk_end = min(chunk0 + CH, col_end);
-        float raw[G][8];
-        rhs_load<G>(a, w, chunk0, chunk_end, kk, rhs_lane, raw);
+        if (!F32) {
+            rhs_load<G>(a, w, chunk0, chunk_end, kk, rhs_lane, raw);
+        }
         for (int c0 = chunk0; c0 < chunk_end; c0 += 32) {
             const int off = c0 - chunk0 + 8 * kk;
             float x2v[8], cb[8], sb[8];
@@ -919,6 +929,7 @@ __device__ __forceinline__ void fwd_table_body(const FwdArgs& a, float* lds, con
     bool tabulated = false;
     for (; chunk0 < col_end; chunk0 += CH) {
         tabulated = true;
+        request_first(chunk0);
         if (!build(chunk0, true)) {
             break;
         }
@@ -927,6 +938,7 @@ __device__ __forceinline__ void fwd_table_body(const FwdArgs& a, float* lds, con
     }
     for (; chunk0 < col_end; chunk0 += CH) {
         if (!tabulated) {
+            request_first(chunk0);
             build(chunk0, false);
         }
         tabulated = false;
@@ -1062,7 +1074,7 @@ __global__ void __launch_bounds__(64 * KM_GROUP_WAVES, 3) fwd_table_f16_grouped(
 }
 
 template <int KT>
-__global__ void __launch_bounds__(64 * KM_GROUP_WAVES, 3) fwd_table_f32_grouped(const FwdArgs a) {
+__global__ void __launch_bounds__(64 * KM_GROUP_WAVES, 4) fwd_table_f32_grouped(const FwdArgs a) {
     extern __shared__ float lds[];
     fwd_table_grouped_kernel<KT, true>(a, lds);
 }

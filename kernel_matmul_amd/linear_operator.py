@@ -255,24 +255,27 @@ class KernelMatmulLinearOperator(LinearOperator):
 
     # -- helpers -------------------------------------------------------------------------
     def _get_args_for_native(self, batch_shape) -> tuple[Tensor, Tensor, Tensor, Tensor, Tensor]:
-        """The constructor tensors as stride-0 views of ``batch_shape`` (kept for the last shape
-        asked for: solvers call with the same one over and over)."""
+        """The constructor tensors as stride-0 views of ``batch_shape``.  The views of the tensors
+        that carry no gradient (coordinates and pattern) are kept for the last shape asked for:
+        solvers call with the same one over and over.  ``params`` is widened on every call, so
+        the view belongs to the autograd mode of that call (a view made under ``no_grad`` or
+        ``inference_mode`` would cut later calls off from the hyper-parameters' gradient)."""
         batch_shape = tuple(batch_shape)
-        if self._native_args is not None and self._native_args[0] == batch_shape:
-            return self._native_args[1]
 
         def widen(t: Tensor, trailing: int) -> Tensor:
             return t.expand(*batch_shape, *t.shape[-trailing:])
 
-        args = (
-            widen(self._x1.squeeze(-1), 1),
-            widen(self._x2.squeeze(-1), 1),
-            widen(self._params, 1),
-            widen(self._start, 1),
-            widen(self._end, 1),
-        )
-        self._native_args = (batch_shape, args)
-        return args
+        if self._native_args is None or self._native_args[0] != batch_shape:
+            fixed = (
+                widen(self._x1.detach().squeeze(-1), 1),
+                widen(self._x2.detach().squeeze(-1), 1),
+                widen(self._start, 1),
+                widen(self._end, 1),
+            )
+            self._native_args = (batch_shape, fixed)
+        x1, x2, start, end = self._native_args[1]
+        params = self._params if tuple(self._params.shape[:-1]) == batch_shape else widen(self._params, 1)
+        return x1, x2, params, start, end
 
     def _transposed_ranges(self, batch_shape=None) -> tuple[Tensor, Tensor]:
         """Pattern of K^T, computed once per operator (the check that the pattern is block

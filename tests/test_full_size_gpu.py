@@ -67,6 +67,8 @@ def _banded_matmul_oracle(kernel, h, rhs, batch_items=None):
     x = h["x"]
     n = x.shape[0]
     rhs = np.asarray(rhs, dtype=np.float64)
+    if rhs.ndim == 3 and batch_items is not None:
+        rhs = rhs[batch_items]
     out = np.zeros((nb, n, rhs.shape[-1]))
     for blk in range(len(h["start"])):
         r0, r1 = blk * 128, min(blk * 128 + 128, n)
@@ -75,7 +77,7 @@ def _banded_matmul_oracle(kernel, h, rhs, batch_items=None):
             continue
         kb = oracle.kernel_matrix(kernel, np.broadcast_to(x[r0:r1], (nb, r1 - r0)),
                                   np.broadcast_to(x[s:e], (nb, e - s)), params)
-        seg = rhs[s:e] if rhs.ndim == 2 else (rhs[:, s:e] if batch_items is None else rhs[batch_items][:, s:e])
+        seg = rhs[s:e] if rhs.ndim == 2 else rhs[:, s:e]
         out[:, r0:r1] = kb @ seg
     return out
 
@@ -99,6 +101,7 @@ def _banded_param_grad_oracle(kernel, h, left, right, batch_items):
     x = h["x"]
     n = x.shape[0]
     right = np.asarray(right, dtype=np.float64)
+    left = np.asarray(left[batch_items], dtype=np.float64)
     grad = np.zeros((nb, params.shape[-1]))
     for blk in range(len(h["start"])):
         r0, r1 = blk * 128, min(blk * 128 + 128, n)
@@ -107,7 +110,7 @@ def _banded_param_grad_oracle(kernel, h, left, right, batch_items):
             continue
         g = oracle.kernel_matrix_grad(kernel, np.broadcast_to(x[r0:r1], (nb, r1 - r0)),
                                       np.broadcast_to(x[s:e], (nb, e - s)), params)
-        coeff = np.asarray(left[batch_items][:, r0:r1], dtype=np.float64) @ right[s:e].T
+        coeff = left[:, r0:r1] @ right[s:e].T
         grad += np.einsum("bij,bpij->bp", coeff, g)
     return grad
 
@@ -155,6 +158,24 @@ def test_forward_every_row_block_against_oracle(name, variant):
     tol = 1e-5 + 1e-4 * np.abs(expected)
     worst = np.unravel_index(np.argmax(err - tol), err.shape)
     assert np.all(err <= tol), (name, variant, worst, err[worst], expected[worst])
+
+
+@pytest.mark.parametrize("variant", [None, "mfma_f32"])
+def test_c5_every_row_block_of_two_batch_items_against_oracle(variant):
+    """Benchmark configuration 5 (n = 10^6, 32 rhs columns: the table kernels with two groups of
+    rhs columns): every output element of two of the eight batch items against the banded
+    float64 oracle."""
+    kernel, n, batch, k, a, h = _build("c5")
+    items = np.array([1, 6])
+    out = _matmul(kernel, a, variant=variant)[items].cpu().double().numpy()
+    key = ("c5", tuple(items))
+    if key not in _FORWARD_ORACLE_CACHE:
+        _FORWARD_ORACLE_CACHE[key] = _banded_matmul_oracle(kernel, h, h["rhs"], batch_items=items)
+    expected = _FORWARD_ORACLE_CACHE[key]
+    err = np.abs(out - expected)
+    tol = 1e-5 + 1e-4 * np.abs(expected)
+    worst = np.unravel_index(np.argmax(err - tol), err.shape)
+    assert np.all(err <= tol), (variant, worst, err[worst], expected[worst])
 
 
 @pytest.mark.parametrize("name,group_tail,halves", [("headline", 0, None), ("headline", 97, None),
@@ -229,7 +250,7 @@ def test_c3_rhs_and_param_gradients_through_the_operator():
 
 def test_c4_bilinear_derivative_against_oracle():
     """Benchmark configuration 4: bilinear derivative, spectral, n = 100000, batch 16, 4 vector
-    columns; the full sums of four batch items against the banded float64 oracle."""
+    columns; the full sums of all sixteen batch items against the banded float64 oracle."""
     kernel, n, batch, k, a, h = _build("c4")
     g = torch.Generator().manual_seed(6)
     left = torch.randn(batch, n, k, generator=g).to(a["x"].device)
@@ -237,7 +258,7 @@ def test_c4_bilinear_derivative_against_oracle():
     got = load_native("bilinear_derivative",
                       BilinearDerivativeConfiguration(kernel).make_config(args)).call(*args)
     assert got.shape == (batch, 3)
-    items = np.array([0, 5, 10, 15])
+    items = np.arange(batch)
     expected = _banded_param_grad_oracle(kernel, h, left.cpu().numpy(), h["rhs"], items)
     tol = 1e-5 + 1e-4 * np.abs(expected).max(axis=-1, keepdims=True)
     err = np.abs(got.cpu().double().numpy()[items] - expected)

@@ -48,13 +48,35 @@ def test_widened_constructor_tensors_are_views_kept_for_the_last_batch_shape():
     start, end = make_ranges(1.0, x.squeeze(-1))
     op = KernelMatmulLinearOperator(x, x, params, start, end, kernel_type="rbf")
     first = op._get_args_for_native(torch.Size((4,)))
-    assert op._get_args_for_native((4,)) is first
+    second = op._get_args_for_native((4,))
+    assert all(t is s for t, s in zip(first, second))
     assert all(t.untyped_storage().data_ptr() == s.untyped_storage().data_ptr()
                for t, s in zip(first, (x, x, params, start, end)))
     wider = op._get_args_for_native((2, 4))
-    assert wider is not first and wider[2].shape == (2, 4, 2) and wider[2].stride(0) == 0
+    assert wider[0] is not first[0] and wider[2].shape == (2, 4, 2) and wider[2].stride(0) == 0
     again = op._get_args_for_native((4,))
     assert [t.shape for t in again] == [t.shape for t in first]
+
+
+def test_widened_params_follow_the_autograd_mode_of_each_call():
+    """A first call under no_grad (or inference_mode) must not cut later calls off from the
+    hyper-parameters: the widened view of params is made per call, only the gradient-free
+    tensors are kept."""
+    x = torch.sort(torch.rand(300, 1), dim=0)[0]
+    start, end = make_ranges(1.0, x.squeeze(-1))
+    for first_mode in (torch.no_grad, torch.inference_mode):
+        params = torch.ones(2, requires_grad=True)
+        op = KernelMatmulLinearOperator(x, x, params, start, end, kernel_type="rbf")
+        for shape in ((), (3,)):
+            with first_mode():
+                quiet = op._get_args_for_native(shape)
+            live = op._get_args_for_native(shape)
+            assert live[2].requires_grad and not live[2].is_inference()
+            assert shape == () or live[2].grad_fn is not None  # () is the operator's own shape: no new view
+            assert live[0] is quiet[0] and live[3] is quiet[3]
+            params.grad = None
+            (live[2] * torch.arange(1.0, 3.0)).sum().backward()
+            assert torch.equal(params.grad, torch.arange(1.0, 3.0) * max(1, int(np.prod(shape))))
 
 
 def _make_operator(kernel_type, batch, m, n, device, square, requires_grad=False):
@@ -127,6 +149,25 @@ def test_autograd_params_and_rhs(kernel_type, square):
     dense = _dense(kernel_type, a, batch)
     expected_rhs = np.swapaxes(dense, -1, -2) @ weight.cpu().double().numpy()
     np.testing.assert_allclose(rhs.grad.cpu().numpy(), expected_rhs, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.gpu
+def test_params_gradient_after_a_first_call_without_grad():
+    device = torch.device("cuda:0")
+    op, params, a = _make_operator("spectral", (2,), 300, 300, device, True, requires_grad=True)
+    rhs = torch.randn(2, 300, 4, device=device)
+    weight = torch.randn(2, 300, 4, device=device)
+    with torch.no_grad():
+        quiet = op._matmul(rhs)
+    out = op._matmul(rhs)
+    assert torch.equal(out, quiet)
+    (out * weight).sum().backward()
+    bc = lambda v: np.broadcast_to(v, (2, *v.shape))
+    expected = oracle.param_grad("spectral", bc(a["x1"]), bc(a["x2"]), weight.cpu().numpy(), rhs.cpu().numpy(),
+                                 a["params"], bc(a["start"]), bc(a["end"]))
+    scale = np.abs(expected).max(axis=-1, keepdims=True)
+    assert params.grad is not None
+    assert np.all(np.abs(params.grad.cpu().numpy() - expected) <= 1e-5 + 1e-4 * scale)
 
 
 @pytest.mark.gpu

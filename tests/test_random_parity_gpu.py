@@ -9,7 +9,10 @@ Tolerance of the forward result, per element: 1e-5 max|rhs| + 1e-4 |expected| + 
 (fp32 evaluation and accumulation), plus, for the oscillating kernels, the fp32 rounding of the
 phase f * d: one ulp of the largest phase times the envelope (Gaussian factor alone) @ |rhs| — the
 error a product formed in fp32 has, in the reference's kernels as much as here.  Gradients: 1e-4
-of the largest component + 2e-5 of sum |coefficient| |dK/dtheta|.
+of the largest component + 8e-6 of sum |coefficient| |dK/dtheta| (twice what the feature form of
+the gradient kernels measures against float64) plus, for the oscillating kernels, the same one ulp
+of every pair's phase: sum |coefficient| |change of dK/dtheta| when the frequency (the period)
+moves by a relative 2^-23, taken from the float64 oracle by a finite difference.
 """
 import random
 
@@ -72,7 +75,7 @@ def _draw(rng):
                 rows_per_wave=rows_per_wave, splits=splits, left=left, right=right)
 
 
-@pytest.mark.parametrize("seed", [2, 4, 5])
+@pytest.mark.parametrize("seed", [1, 2, 3])
 def test_random_cases_against_oracle(seed):
     rng = random.Random(seed)
     torch.manual_seed(seed)
@@ -116,6 +119,12 @@ def test_random_cases_against_oracle(seed):
         mask = oracle.range_mask(start, end, x1.shape[-1], x2.shape[-1])
         coeff = np.abs(left.astype(np.float64) @ np.swapaxes(right.astype(np.float64), -1, -2))
         size = np.sum(np.where(mask, coeff, 0.0)[..., None, :, :] * terms, axis=(-2, -1))
-        tol_g = 1e-4 * np.abs(expected_g).max(axis=-1, keepdims=True) + 2e-5 * size + 1e-6
+        tol_g = 1e-4 * np.abs(expected_g).max(axis=-1, keepdims=True) + 8e-6 * size + 1e-6
+        if kt != "rbf":
+            eta = 2.0 ** -20
+            moved = params.astype(np.float64).copy()
+            moved[..., 1 if kt == "spectral" else 2] *= 1.0 + eta
+            change = np.abs(oracle.kernel_matrix_grad(kt, x1, x2, moved) - oracle.kernel_matrix_grad(kt, x1, x2, params))
+            tol_g = tol_g + np.sum(np.where(mask, coeff, 0.0)[..., None, :, :] * change, axis=(-2, -1)) * (2.0 ** -23 / eta)
         assert np.all(np.isfinite(got)), what
         assert np.all(np.abs(got - expected_g) <= tol_g), (what, float(np.max(np.abs(got - expected_g) / tol_g)))
