@@ -55,6 +55,27 @@ SPIN_UP_MS = 100.0
 TRAFFIC_SOURCE = "profiles/fwd_table_f16_grouped_headline_counters.md"
 MEASURED_TRAFFIC_BYTES = {"headline": 58640794}
 
+# Share of the kernel's cycles in which the SIMDs' VALU is busy (SQ_ACTIVE_INST_VALU x 4 / SIMD
+# cycles), from the offline counter runs summarised under profiles/ (not measured by this script).
+VALU_BUSY = {
+    "headline": (0.75, "profiles/fwd_table_f16_grouped_headline_counters.md"),
+    "c1": (0.10, "profiles/fwd_table_f16_midsize_c1_c2_c3_profile.md"),
+    "c2": (0.43, "profiles/fwd_table_f16_midsize_c1_c2_c3_profile.md"),
+    "c3_rhs_grad": (0.36, "profiles/fwd_table_f16_midsize_c1_c2_c3_profile.md"),
+    "c4": (0.73, "profiles/param_grad_features_c4_profile.md"),
+    "c5": (0.86, "profiles/forward_c5_and_reference_recipe_profile.md"),
+    "ref_example": (0.43, "profiles/forward_c5_and_reference_recipe_profile.md"),
+}
+
+
+def pipe_of(kernel_description: str) -> str:
+    """Which pipes do the work of the kernel the library says it launches."""
+    if "fwd_valu" in kernel_description:
+        return "valu"
+    if "f32" in kernel_description or "param_grad_partial" in kernel_description:
+        return "valu+mfma_f32"
+    return "valu+mfma_f16"
+
 FLOPS_PER_PAIR = {"rbf": lambda k: 5 + 2 * k, "spectral": lambda k: 8 + 2 * k,
                   "locally_periodic": lambda k: 10 + 2 * k}
 GRAD_FLOPS_PER_PAIR = {"rbf": lambda c: 6 + 2 * c + 2 * 2, "spectral": lambda c: 14 + 2 * c + 2 * 3}
@@ -217,8 +238,13 @@ class Prepared:
             "wall_ms_per_call": t["wall_ms"],
             "pairs_per_s_kernel": self.pairs / (t["kernel_ms"] * 1e-3),
             "pairs_per_s_wall": self.pairs / (t["wall_ms"] * 1e-3),
-            "frac_of_fp32_peak": flops / (t["kernel_ms"] * 1e-3) / 1e12 / PEAK_FP32_TFLOPS,
-            "frac_of_fp32_peak_back_to_back": flops / (t["stream_ms"] * 1e-3) / 1e12 / PEAK_FP32_TFLOPS,
+            # nominal flops (direct evaluation, fp32 contraction) per second over the fp32 peak: a
+            # normalised throughput, above 1 where the contraction runs on the fp16 matrix pipe
+            "algorithmic_frac_vs_fp32_peak": flops / (t["kernel_ms"] * 1e-3) / 1e12 / PEAK_FP32_TFLOPS,
+            "algorithmic_frac_vs_fp32_peak_back_to_back": flops / (t["stream_ms"] * 1e-3) / 1e12 / PEAK_FP32_TFLOPS,
+            "pipe": pipe_of(self.kernel),
+            "valu_busy": VALU_BUSY.get(self.name, (None, None))[0],
+            "valu_busy_source": VALU_BUSY.get(self.name, (None, None))[1],
         }
 
 
@@ -301,6 +327,11 @@ def main() -> int:
         torch.cuda.synchronize()
         del src, dst
 
+    default_run = args.workload == "headline" and args.batch is None and args.variant in ("auto", "mfma_f16")
+    traffic = MEASURED_TRAFFIC_BYTES["headline"] if default_run else None
+
+    # The same steps right after the warm-up, before the GPU has raised its clocks.
+    cold = main_run.measure(args.steps, 0, 0.0)
     # Whole-step wall time of the timed region and, on the launch stream, the event time over the
     # region and around single launches.
     timing = main_run.measure(args.steps, 0, args.spin_up_ms)
@@ -311,8 +342,6 @@ def main() -> int:
     achieved_tflops = pairs * flops_per_pair / (kernel_ms_avg * 1e-3) / 1e12
     back_to_back_tflops = pairs * flops_per_pair / (timing["stream_ms"] * 1e-3) / 1e12
 
-    default_run = args.workload == "headline" and args.batch is None and args.variant in ("auto", "mfma_f16")
-    traffic = MEASURED_TRAFFIC_BYTES["headline"] if default_run else None
 
     result = {
         "metric": "kernel-pair evaluations/s (sparse spectral K@rhs, n=100k, k=16, 1 MI355X)",
@@ -327,8 +356,8 @@ def main() -> int:
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32 in/out, K evaluated in f32 on the VALU; contraction: split-fp16 MFMA (hi+lo, 22 bits per "
-                 "factor) with f32 accumulation" if args.variant in ("auto", "mfma_f16", "mfma_f16_direct", "block")
-                 else "f32",
+                 "factor) with f32 accumulation (roofline.fp32_mfma_variant: the same with every product in f32)"
+                 if args.variant in ("auto", "mfma_f16", "mfma_f16_direct", "block") else "f32",
         "data": "synthetic",
         "config": {
             "workload": w["label"],
@@ -357,6 +386,19 @@ def main() -> int:
                 "achieved": back_to_back_tflops,
                 "frac": back_to_back_tflops / PEAK_FP32_TFLOPS,
             },
+            "cold": {
+                "what": "the same steps timed right after --warmup, without the spin-up launches",
+                "ms_per_step": cold["wall_ms"],
+                "pairs_per_s": pairs / (cold["wall_ms"] * 1e-3),
+                "kernel_ms_avg": cold["kernel_ms"],
+                "frac": pairs * flops_per_pair / (cold["kernel_ms"] * 1e-3) / 1e12 / PEAK_FP32_TFLOPS,
+            },
+            "pipe": pipe_of(main_run.kernel),
+            "valu_busy": VALU_BUSY["headline"][0] if default_run else None,
+            "valu_busy_source": VALU_BUSY["headline"][1] if default_run else None,
+            "achieved_is": "nominal flops per pair (8 + 2k: direct evaluation, fp32 contraction) x pairs / kernel "
+                           "time; the kernel launched executes fewer VALU operations per pair (separable exponent, "
+                           "tabulated phases) and contracts on the matrix pipe named in `pipe`",
             "note": "bound by VALU issue (kernel evaluation in fp32 + hi/lo split + MFMA issue), priced against "
                     "the fp32 peak (157.3 TFLOP/s vector == fp32 MFMA); flops = pairs * (8 + 2k), one "
                     "transcendental counted as 1.  The contraction itself runs as split-fp16 MFMAs, so frac is "
@@ -365,15 +407,18 @@ def main() -> int:
     }
 
     if default_run:
-        # The same workload with the contraction as a true fp32 MFMA (v_mfma_f32_16x16x4_f32).
+        # The same workload with the contraction as a true fp32 MFMA (v_mfma_f32_16x16x4_f32): K
+        # evaluated in fp32 on the VALU, every product and sum of the contraction in fp32.
         f32_run = Prepared("headline", device, variant="mfma_f32")
         f32_timing = f32_run.measure(max(args.steps // 2, 5), 2)
         f32_ms, f32_out = f32_timing["kernel_ms"], f32_timing["out"]
         result["roofline"]["fp32_mfma_variant"] = {
             "kernel": f32_run.kernel,
+            "pipe": pipe_of(f32_run.kernel),
             "kernel_ms": f32_ms,
             "frac": pairs * flops_per_pair / (f32_ms * 1e-3) / 1e12 / PEAK_FP32_TFLOPS,
             "back_to_back_kernel_ms": f32_timing["stream_ms"],
+            "back_to_back_frac": pairs * flops_per_pair / (f32_timing["stream_ms"] * 1e-3) / 1e12 / PEAK_FP32_TFLOPS,
         }
     else:
         f32_out = None

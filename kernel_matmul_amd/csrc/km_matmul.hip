@@ -458,34 +458,45 @@ __device__ __forceinline__ void f32_step(const float (&x2v)[8], const float (&ra
             bv[g][t] = (SEP && KT == KM_KERNEL_RBF) ? raw[g][t] * cb[t] : raw[g][t];
         }
     }
+    // Two row groups at a time: their entries are evaluated first, then their MFMAs are issued
+    // alternating between the two accumulators.
+    constexpr int RI = R >= 2 ? 2 : 1;
 #pragma unroll
-    for (int r = 0; r < R; r++) {
-        float kv[8];
-        if (SEP) {
-            const float av = (x1v[r] - ref) * kc.s;
-            const float rb = -av * av;
+    for (int r0 = 0; r0 < R; r0 += RI) {
+        float kv[RI][8];
 #pragma unroll
-            for (int t = 0; t < 8; t++) {
-                kv[t] = __builtin_amdgcn_exp2f(__builtin_fmaf(av, x2v[t], rb));
+        for (int q = 0; q < RI; q++) {
+            const int r = r0 + q;
+            if (SEP) {
+                const float av = (x1v[r] - ref) * kc.s;
+                const float rb = -av * av;
+#pragma unroll
+                for (int t = 0; t < 8; t++) {
+                    kv[q][t] = __builtin_amdgcn_exp2f(__builtin_fmaf(av, x2v[t], rb));
+                }
+            } else {
+#pragma unroll
+                for (int t = 0; t < 8; t++) {
+                    const float u = (x1v[r] - x2v[t]) * kc.s;
+                    kv[q][t] = __builtin_amdgcn_exp2f(-u * u);
+                }
             }
-        } else {
+            if (KT == KM_KERNEL_SPECTRAL) {
 #pragma unroll
-            for (int t = 0; t < 8; t++) {
-                const float u = (x1v[r] - x2v[t]) * kc.s;
-                kv[t] = __builtin_amdgcn_exp2f(-u * u);
-            }
-        }
-        if (KT == KM_KERNEL_SPECTRAL) {
-#pragma unroll
-            for (int t = 0; t < 8; t++) {
-                kv[t] *= __builtin_fmaf(sa[r], sb[t], ca[r] * cb[t]);
+                for (int t = 0; t < 8; t++) {
+                    kv[q][t] *= __builtin_fmaf(sa[r], sb[t], ca[r] * cb[t]);
+                }
             }
         }
 #pragma unroll
         for (int t = 0; t < 8; t++) {
 #pragma unroll
-            for (int g = 0; g < G; g++) {
-                acc[r][g] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv[t], bv[g][t], acc[r][g], 0, 0, 0);
+            for (int q = 0; q < RI; q++) {
+#pragma unroll
+                for (int g = 0; g < G; g++) {
+                    acc[r0 + q][g] =
+                        __builtin_amdgcn_mfma_f32_16x16x4f32(kv[q][t], bv[g][t], acc[r0 + q][g], 0, 0, 0);
+                }
             }
         }
     }
@@ -908,7 +919,22 @@ __device__ __forceinline__ void fwd_table_body(const FwdArgs& a, float* lds, con
             const float ref = SEP ? tab_ref[off >> 3] : 0.0f;
             // (chunks that cannot take the separable form evaluate the whole kernel directly)
             if constexpr (F32) {
+                // The next step's rhs operand is requested before this step is evaluated.
+                float rawn[G][8];
+                if (c0 + 32 < chunk_end) {
+                    rhs_load<G>(a, w, c0 + 32, chunk_end, kk, rhs_lane, rawn);
+                }
                 f32_step<KT, G, R, SEP>(x2v, raw, x1v, kc, acc, ref, cb, sb, row_cos, row_sin);
+                if (c0 + 32 < chunk_end) {
+#pragma unroll
+                    for (int g = 0; g < G; g++) {
+#pragma unroll
+                        for (int t = 0; t < 8; t++) {
+                            raw[g][t] = rawn[g][t];
+                        }
+                    }
+                }
+                continue;
             } else {
                 f16_step<PAIRCOS ? KM_KERNEL_SPECTRAL : KM_KERNEL_RBF, G, R, KS, SEP, GE / G, SEP && !PHASE,
                          PAIRCOS && SEP>(x2v, raw, x1v, kc, colmask, shift, scale, acc, ref, cb, sb, row_phase);
