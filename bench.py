@@ -42,6 +42,9 @@ WORKLOADS = {
                label="spectral bilinear_derivative n=100000 d=4 batch=16 cutoff=6*l_max"),
     "c5": dict(kernel="spectral", n=1_000_000, extent=100_000.0, batch=8, k=32, cutoff_l=5.0, seed=1005,
                label="spectral K@rhs n=1000000 k=32 batch=8 cutoff=5*l_max"),
+    # gradient at the headline's size with 8 vector columns (beyond the feature form's widths)
+    "grad_c8": dict(kernel="spectral", n=100_000, extent=10_000.0, batch=8, k=8, cutoff_l=6.0, seed=1006, op="param_grad",
+                    label="spectral bilinear_derivative n=100000 d=8 batch=8 cutoff=6*l_max"),
     # the reference's own benchmark recipe (examples/matmul.py:61-82 there)
     "ref_example": dict(kernel="rbf", n=65_536, extent=65_536 / 24.0, batch=1, k=64, cutoff_abs=10.0, seed=0,
                         label="rbf K@rhs n=65536 k=64 batch=1 x~U[0,n/24) cutoff=10 params=1+0.01*N(0,1)"),

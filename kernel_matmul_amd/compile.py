@@ -103,7 +103,7 @@ class NativeModule:
         options = _native.LaunchOptions()
         col_blocks = self.defines.get("MATMUL_COL_BLOCKS")
         if col_blocks is not None and col_blocks > 1:
-            options.col_splits = max(s for s in (1, 2, 4, 8) if s <= col_blocks)
+            options.col_splits = min(int(col_blocks), 8)
         variant = self.defines.get("MATMUL_VARIANT")
         if variant is not None:
             options.variant = {"auto": 0, "valu": 1, "mfma": 2, "mfma_f32": 2, "mfma_f16": 3, "mfma_f16_direct": 4,

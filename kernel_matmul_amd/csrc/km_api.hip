@@ -193,8 +193,8 @@ static int make_plan(const MatmulProblem& p, const km_launch_options* opt, Matmu
     int S = 1;
     if (opt && opt->col_splits != 0) {
         S = opt->col_splits;
-        if (S != 1 && S != 2 && S != 4 && S != 8) {
-            return fail(KM_ERR_INVALID_ARGUMENT, "km_matmul: col_splits must be 1, 2, 4 or 8");
+        if (S < 1 || S > 8) {
+            return fail(KM_ERR_INVALID_ARGUMENT, "km_matmul: col_splits must be 1 to 8");
         }
     } else if (table && !two_per_simd) {
         // Table kernels: the share count that leaves the fullest SIMD the least work,

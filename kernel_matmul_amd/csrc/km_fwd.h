@@ -162,6 +162,10 @@ struct WaveView {
     int range_end;
 };
 
+// FAST: take the short way when the batch shape has collapsed to at most one dimension (small
+// launches, where the scalar prologue is a visible part of a wavefront's life; the large grouped
+// launches measure 2 % slower with the extra branch and keep the general code).
+template <bool FAST = false>
 __device__ __forceinline__ WaveView wave_view(const FwdArgs& a, long long item, int chunks_per_block,
                                               int* chunk_in_block) {
     WaveView w;
@@ -169,16 +173,34 @@ __device__ __forceinline__ WaveView wave_view(const FwdArgs& a, long long item, 
     const int chunk = (int)(item / a.num_batches);
     w.row_block = chunk / chunks_per_block;
     *chunk_in_block = chunk % chunks_per_block;
-    int bidx[KM_MAX_BATCH_RANK];
-    batch_multi_index(a.batch, w.b, bidx);
-    w.x1 = a.x1 + batch_offset(a.batch, a.x1_bs, bidx);
-    w.x2 = a.x2 + batch_offset(a.batch, a.x2_bs, bidx);
-    w.rhs = a.rhs + batch_offset(a.batch, a.rhs_bs, bidx);
-    w.params = a.params + batch_offset(a.batch, a.params_bs, bidx);
+    long long off_x1, off_x2, off_rhs, off_params, off_start, off_end;
+    if (FAST && a.batch.rank <= 1) {
+        // The usual case after the host has collapsed the batch dimensions: one stride per
+        // tensor, no division chain.
+        off_x1 = w.b * a.x1_bs.s[0];
+        off_x2 = w.b * a.x2_bs.s[0];
+        off_rhs = w.b * a.rhs_bs.s[0];
+        off_params = w.b * a.params_bs.s[0];
+        off_start = w.b * a.start_bs.s[0];
+        off_end = w.b * a.end_bs.s[0];
+    } else {
+        int bidx[KM_MAX_BATCH_RANK];
+        batch_multi_index(a.batch, w.b, bidx);
+        off_x1 = batch_offset(a.batch, a.x1_bs, bidx);
+        off_x2 = batch_offset(a.batch, a.x2_bs, bidx);
+        off_rhs = batch_offset(a.batch, a.rhs_bs, bidx);
+        off_params = batch_offset(a.batch, a.params_bs, bidx);
+        off_start = batch_offset(a.batch, a.start_bs, bidx);
+        off_end = batch_offset(a.batch, a.end_bs, bidx);
+    }
+    w.x1 = a.x1 + off_x1;
+    w.x2 = a.x2 + off_x2;
+    w.rhs = a.rhs + off_rhs;
+    w.params = a.params + off_params;
     // Clamped to the valid columns: a symmetric pattern over fewer points than one block
     // reports end = block size > n (native/ranges/ranges.cpp:82-93 of the reference).
-    w.range_start = max(a.start[batch_offset(a.batch, a.start_bs, bidx) + w.row_block * a.start_s], 0);
-    w.range_end = min(a.end[batch_offset(a.batch, a.end_bs, bidx) + w.row_block * a.end_s], a.n);
+    w.range_start = max(a.start[off_start + w.row_block * a.start_s], 0);
+    w.range_end = min(a.end[off_end + w.row_block * a.end_s], a.n);
     return w;
 }
 

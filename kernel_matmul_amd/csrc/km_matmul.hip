@@ -1023,7 +1023,7 @@ __device__ __forceinline__ void fwd_table_kernel(const FwdArgs& a, float* lds) {
         return;
     }
     int chunk_in_block;
-    const WaveView w = wave_view(a, item, a.chunks_per_block, &chunk_in_block);
+    const WaveView w = wave_view<true>(a, item, a.chunks_per_block, &chunk_in_block);
     // (the wavefront index is wave-uniform by construction; saying so keeps what is derived from
     // it in scalar registers)
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);

@@ -199,15 +199,29 @@ __device__ __forceinline__ bool grad_item(const GradArgs& a, int rows_per_item, 
     const int row_block = chunk / chunks_per_block;
     g->row0 = row_block * KM_BLOCK_SIZE + (chunk % chunks_per_block) * rows_per_item;
 
-    int bidx[KM_MAX_BATCH_RANK];
-    batch_multi_index(a.batch, g->b, bidx);
-    g->x1 = a.x1 + batch_offset(a.batch, a.x1_bs, bidx);
-    g->x2 = a.x2 + batch_offset(a.batch, a.x2_bs, bidx);
-    g->left = a.left + batch_offset(a.batch, a.left_bs, bidx);
-    g->right = a.right + batch_offset(a.batch, a.right_bs, bidx);
-    g->params = a.params + batch_offset(a.batch, a.params_bs, bidx);
-    int range_start = a.start[batch_offset(a.batch, a.start_bs, bidx) + row_block * a.start_s];
-    int range_end = a.end[batch_offset(a.batch, a.end_bs, bidx) + row_block * a.end_s];
+    long long off_start, off_end;
+    if (a.batch.rank <= 1) {
+        // The usual case after the host has collapsed the batch dimensions: one stride per tensor.
+        g->x1 = a.x1 + g->b * a.x1_bs.s[0];
+        g->x2 = a.x2 + g->b * a.x2_bs.s[0];
+        g->left = a.left + g->b * a.left_bs.s[0];
+        g->right = a.right + g->b * a.right_bs.s[0];
+        g->params = a.params + g->b * a.params_bs.s[0];
+        off_start = g->b * a.start_bs.s[0];
+        off_end = g->b * a.end_bs.s[0];
+    } else {
+        int bidx[KM_MAX_BATCH_RANK];
+        batch_multi_index(a.batch, g->b, bidx);
+        g->x1 = a.x1 + batch_offset(a.batch, a.x1_bs, bidx);
+        g->x2 = a.x2 + batch_offset(a.batch, a.x2_bs, bidx);
+        g->left = a.left + batch_offset(a.batch, a.left_bs, bidx);
+        g->right = a.right + batch_offset(a.batch, a.right_bs, bidx);
+        g->params = a.params + batch_offset(a.batch, a.params_bs, bidx);
+        off_start = batch_offset(a.batch, a.start_bs, bidx);
+        off_end = batch_offset(a.batch, a.end_bs, bidx);
+    }
+    int range_start = a.start[off_start + row_block * a.start_s];
+    int range_end = a.end[off_end + row_block * a.end_s];
     range_start = max(range_start, 0);
     range_end = min(range_end, a.n);
     // Column share of this wavefront, in whole steps of col_step columns.
