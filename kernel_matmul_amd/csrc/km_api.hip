@@ -252,8 +252,34 @@ static int make_plan(const MatmulProblem& p, const km_launch_options* opt, Matmu
             }
         }
     }
-    if (!(table && G == 1 && R == 8 && S == 1)) {
+    // Mid-size problems through the table kernel in 64-row items (the launch table's choice when
+    // 128-row items would not fill the SIMDs once): whole rounds of one item per SIMD go one item
+    // per wavefront, the remainder of every XCD is split by columns and dispatched last.  Measured
+    // (spectral, k = 16) against column shares for every item: n = 20000, batch 5 (197 items per
+    // XCD) 26.0 against 32.6 us, batch 6 (236) 30.0 against 33.0 us; n = 50000, batch 2 (196) 24.4
+    // against 26.0 us; n = 1e5, batch 1 (196) 23.6 against 25.0 us.  With few items beyond one per
+    // SIMD the long wavefronts run alone and cannot hide their own latencies (n = 20000, batch 4:
+    // 157 per XCD, 26.1 against 22.7 us), hence the lower bound on the remainder.
+    const bool mid = variant == KM_VARIANT_MFMA_F16 && table && G == 1 && R == 4 && plan->tail_balance &&
+                     !(opt && (opt->col_splits != 0 || opt->rows_per_wave != 0));
+    if (mid && plan->group_tail < 0) {
+        const long long per_xcd = (row_blocks * 2 * p.num_batches + KM_NUM_XCD - 1) / KM_NUM_XCD;
+        if (per_xcd >= 128 + 48) {
+            plan->group_tail = per_xcd % 128;
+            S = 1;
+            plan->col_splits = 1;
+        }
+    }
+    if (plan->group_tail >= 0 && table && G == 1 && (R == 8 || (R == 4 && variant == KM_VARIANT_MFMA_F16)) &&
+        !(opt && opt->col_splits != 0)) {
+        S = 1;  // an explicit tail asks for the grouped launch
+        plan->col_splits = 1;
+    }
+    if (!(table && G == 1 && S == 1 && (R == 8 || (R == 4 && variant == KM_VARIANT_MFMA_F16)))) {
         plan->group_tail = -1;
+    }
+    if (R == 4) {
+        plan->group_tail_halves = 0;
     }
     // The very last of the split items also run as two halves of 64 rows (pieces of an eighth of
     // an item; they repeat the column-side work).
@@ -499,6 +525,13 @@ int km_matmul_describe(int kernel_type, int64_t num_batches, int64_t m, int64_t 
                                    : (plan.variant == KM_VARIANT_MFMA_F32
                                           ? "km::fwd_table_f32"
                                           : (plan.variant == KM_VARIANT_MFMA_F16 ? "km::fwd_table_f16" : "km::fwd_mfma_f16"));
+            if (plan.variant == KM_VARIANT_MFMA_F16 && plan.group_tail >= 0 && plan.row_groups == 4) {
+                snprintf(text, text_bytes,
+                         "%s_grouped64<%s>: 64 rows per wavefront, 4 wavefronts per workgroup, the last %lld "
+                         "items of each XCD split by columns over a workgroup",
+                         name, kt, plan.group_tail);
+                break;
+            }
             if ((plan.variant == KM_VARIANT_MFMA_F16 || plan.variant == KM_VARIANT_MFMA_F32) && plan.group_tail >= 0) {
                 snprintf(text, text_bytes,
                          "%s_grouped<%s>: 128 rows per wavefront, 4 wavefronts per workgroup, the "

@@ -1099,6 +1099,40 @@ __global__ void __launch_bounds__(64 * KM_GROUP_WAVES, 3) fwd_table_f16_grouped(
     fwd_table_grouped_kernel<KT, false>(a, lds);
 }
 
+// The same launch shape for mid-size problems, where 128-row items would not fill the SIMDs
+// once: the items are 64-row chunks, one per wavefront in workgroups of four; whatever exceeds
+// whole rounds of one item per SIMD (the last `tail_items` of every XCD) is dispatched last, each
+// split by columns over a workgroup.  A SIMD then runs one long wavefront and a few short ones
+// beside it, where one wavefront per chunk would leave a fifth of the SIMDs with two and column
+// shares for every chunk would put thousands of short-lived wavefronts through the dispatcher.
+template <int KT>
+__global__ void __launch_bounds__(64 * KM_GROUP_WAVES, 4) fwd_table_f16_grouped64(const FwdArgs a) {
+    extern __shared__ float lds[];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const unsigned xcd = blockIdx.x % KM_NUM_XCD;
+    const long long slot = blockIdx.x / KM_NUM_XCD;
+    const long long main_items = a.items_per_xcd - a.tail_items;
+    const long long main_groups = (main_items + KM_GROUP_WAVES - 1) / KM_GROUP_WAVES;
+    const bool split = slot >= main_groups;
+    long long local;
+    if (!split) {
+        local = slot * KM_GROUP_WAVES + wave;
+        if (local >= main_items) {
+            return;
+        }
+    } else {
+        local = main_items + (slot - main_groups);
+    }
+    const long long item = (long long)xcd * a.items_per_xcd + local;
+    if (item >= a.total_items) {
+        return;  // uniform for the workgroup of a split item
+    }
+    int chunk_in_block;
+    const WaveView w = wave_view<true>(a, item, 2, &chunk_in_block);
+    fwd_table_body<KT, 1, 4, false>(a, lds, w, w.row_block * KM_BLOCK_SIZE + 64 * chunk_in_block,
+                                    split ? KM_GROUP_WAVES : 1, split ? wave : 0, wave, true);
+}
+
 template <int KT>
 __global__ void __launch_bounds__(64 * KM_GROUP_WAVES, 4) fwd_table_f32_grouped(const FwdArgs a) {
     extern __shared__ float lds[];
@@ -1307,6 +1341,23 @@ hipError_t launch_matmul(const MatmulProblem& p, const MatmulPlan& plan, hipStre
             case KM_KERNEL_SPECTRAL: return launch_valu<KM_KERNEL_SPECTRAL>(a, plan.k_chunk, grid_x, grid_y, stream);
             default: return launch_valu<KM_KERNEL_LOCALLY_PERIODIC>(a, plan.k_chunk, grid_x, grid_y, stream);
         }
+    }
+    if (plan.variant == KM_VARIANT_MFMA_F16 && plan.group_tail >= 0 && plan.row_groups == 4 && plan.col_splits == 1 &&
+        plan.k_chunk == 16 && p.kernel_type != KM_KERNEL_LOCALLY_PERIODIC) {
+        // 64-row items (a.total_items / a.items_per_xcd already count them)
+        a.tail_items = (int)(plan.group_tail < a.items_per_xcd ? plan.group_tail : a.items_per_xcd);
+        a.tail_half_items = 0;
+        const long long main_groups = (a.items_per_xcd - a.tail_items + KM_GROUP_WAVES - 1) / KM_GROUP_WAVES;
+        const unsigned gx = (unsigned)((main_groups + a.tail_items) * KM_NUM_XCD);
+        const size_t table = (size_t)KM_GROUP_WAVES * KM_PHASE_TABLE_FLOATS * sizeof(float);
+        if (p.kernel_type == KM_KERNEL_SPECTRAL) {
+            hipLaunchKernelGGL((fwd_table_f16_grouped64<KM_KERNEL_SPECTRAL>), dim3(gx, grid_y, 1),
+                               dim3(64 * KM_GROUP_WAVES, 1, 1), table, stream, a);
+        } else {
+            hipLaunchKernelGGL((fwd_table_f16_grouped64<KM_KERNEL_RBF>), dim3(gx, grid_y, 1),
+                               dim3(64 * KM_GROUP_WAVES, 1, 1), table, stream, a);
+        }
+        return hipGetLastError();
     }
     if ((plan.variant == KM_VARIANT_MFMA_F16 || plan.variant == KM_VARIANT_MFMA_F32) && plan.group_tail >= 0 &&
         plan.row_groups == 8 && plan.col_splits == 1 && plan.k_chunk == 16 &&

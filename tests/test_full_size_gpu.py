@@ -178,22 +178,27 @@ def test_c5_every_row_block_of_two_batch_items_against_oracle(variant):
     assert np.all(err <= tol), (variant, worst, err[worst], expected[worst])
 
 
-@pytest.mark.parametrize("name,group_tail,halves", [("headline", 0, None), ("headline", 97, None),
-                                                    ("headline", 97, 0), ("headline", 97, 97),
-                                                    ("headline", 10_000, None), ("headline", 10_000, 0),
-                                                    ("c2", 5, None), ("c2", 5, 5), ("c3_rbf", 3, 2)])
-def test_forward_grouped_launch_against_oracle(name, group_tail, halves):
+@pytest.mark.parametrize("name,group_tail,halves,rows", [
+    ("headline", 0, None, 128), ("headline", 97, None, 128), ("headline", 97, 0, 128), ("headline", 97, 97, 128),
+    ("headline", 10_000, None, 128), ("headline", 10_000, 0, 128), ("c2", 5, None, 128), ("c2", 5, 5, 128),
+    ("c3_rbf", 3, 2, 128),
+    # 64-row items (mid-size launches): none, some, the usual remainder and all of them split
+    ("c2", 0, None, 64), ("c2", 29, None, 64), ("c2", 10_000, None, 64), ("c3", 68, None, 64), ("c3_rbf", 7, None, 64)])
+def test_forward_grouped_launch_against_oracle(name, group_tail, halves, rows):
     """Workgroups of four wavefronts: full items one per wavefront, the last `group_tail` items of
     every XCD split by columns between the four wavefronts of a workgroup (fixed-order sum), the
-    last `halves` of them (default: a quarter) also into two workgroups of 64 rows each."""
+    last `halves` of them (default: a quarter) also into two workgroups of 64 rows each.  With 64
+    rows per wavefront the items are 64-row chunks (no halves)."""
     kernel, n, batch, k, a, h = _build(name)
     op_args = (a["x"], a["x"], a["rhs"], a["params"], a["start"], a["end"])
     defines = MatmulSingleConfiguration(kernel).make_config(op_args)
     defines["MATMUL_VARIANT"] = "mfma_f16"
-    defines["MATMUL_ROWS_PER_WAVE"] = 128
+    defines["MATMUL_ROWS_PER_WAVE"] = rows
     defines["MATMUL_GROUP_TAIL"] = group_tail
     if halves is not None:
         defines["MATMUL_GROUP_TAIL_HALVES"] = halves
+    op = load_native("matmul", defines)
+    assert ("grouped64" if rows == 64 else "grouped<") in op.describe(*op_args)
     out = load_native("matmul", defines).call(*op_args)
     again = load_native("matmul", defines).call(*op_args)
     assert torch.equal(out, again)  # fixed reduction order: reproducible

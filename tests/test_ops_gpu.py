@@ -34,7 +34,7 @@ def assert_close(actual: torch.Tensor, expected: np.ndarray, rtol=RTOL, atol=ATO
     )
 
 
-@pytest.mark.parametrize("col_blocks", [1, 2])
+@pytest.mark.parametrize("col_blocks", [1, 2, 3, 7])
 def test_matmul(example_data, col_blocks):
     d = example_data
     args = (d.x1, d.x2, d.rhs, d.params, d.start, d.end)

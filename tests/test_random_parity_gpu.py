@@ -68,7 +68,7 @@ def _draw(rng):
     rhs = torch.randn(*batch, n, k) * rng.choice([1.0, 1e-3, 1e3])
     variant = rng.choice([None, None, None, "mfma_f16", "mfma_f16_direct", "block", "mfma_f32", "mfma_f32_direct", "valu"])
     rows_per_wave = rng.choice([None, None, 16, 32, 64, 128])
-    splits = rng.choice([None, None, 1, 2, 4, 8])
+    splits = rng.choice([None, None, 1, 2, 3, 4, 5, 8])
     c = rng.choice([1, 3, 4, 5, 8, 10, 16])
     left, right = torch.randn(*batch, m, c), torch.randn(*batch, n, c)
     return dict(kt=kt, x1=x1, x2=x2, rhs=rhs, params=params, start=start, end=end, variant=variant,
