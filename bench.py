@@ -62,11 +62,14 @@ MEASURED_TRAFFIC_BYTES = {"headline": 58640794}
 # cycles), from the offline counter runs summarised under profiles/ (not measured by this script).
 VALU_BUSY = {
     "headline": (0.75, "profiles/fwd_table_f16_grouped_headline_counters.md"),
-    "c1": (0.10, "profiles/fwd_table_f16_midsize_c1_c2_c3_profile.md"),
-    "c2": (0.43, "profiles/fwd_table_f16_midsize_c1_c2_c3_profile.md"),
-    "c3_rhs_grad": (0.36, "profiles/fwd_table_f16_midsize_c1_c2_c3_profile.md"),
+    "headline_fp32": (0.46, "profiles/fwd_table_f32_grouped_headline_profile.md"),
+    "c1": (0.12, "profiles/fwd_table_f16_midsize_c1_c2_c3_profile.md"),
+    "c2": (0.44, "profiles/fwd_table_f16_midsize_c1_c2_c3_profile.md"),
+    "c3": (0.51, "profiles/param_grad_partial_c3_and_wide_vectors_profile.md"),
+    "c3_rhs_grad": (0.47, "profiles/fwd_table_f16_midsize_c1_c2_c3_profile.md"),
     "c4": (0.73, "profiles/param_grad_features_c4_profile.md"),
     "c5": (0.86, "profiles/forward_c5_and_reference_recipe_profile.md"),
+    "grad_c8": (0.65, "profiles/param_grad_partial_c3_and_wide_vectors_profile.md"),
     "ref_example": (0.43, "profiles/forward_c5_and_reference_recipe_profile.md"),
 }
 
@@ -418,6 +421,10 @@ def main() -> int:
         result["roofline"]["fp32_mfma_variant"] = {
             "kernel": f32_run.kernel,
             "pipe": pipe_of(f32_run.kernel),
+            "valu_busy": VALU_BUSY["headline_fp32"][0],
+            "mfma_busy": 0.395,
+            "busy_source": VALU_BUSY["headline_fp32"][1] + " (VALU and fp32-MFMA cycles are disjoint on gfx950: "
+                           "together 86 % of the kernel's cycles at batch 8, 95 % at batch 64)",
             "kernel_ms": f32_ms,
             "frac": pairs * flops_per_pair / (f32_ms * 1e-3) / 1e12 / PEAK_FP32_TFLOPS,
             "back_to_back_kernel_ms": f32_timing["stream_ms"],
