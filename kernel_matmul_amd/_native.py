@@ -332,6 +332,10 @@ def describe_matmul(kernel_type: str, num_batches: int, m: int, n: int, k: int,
     return text.value.decode()
 
 
+# device index -> (stream handle, event recorded after the last km_param_grad_static call there)
+_STATIC_SCRATCH_USE: dict = {}
+
+
 def param_grad(kernel_type: str, x1: Tensor, x2: Tensor, left: Tensor, right: Tensor,
                params: Tensor, start: Tensor, end: Tensor, out: Tensor | None = None,
                static_scratch: bool = False) -> Tensor:
@@ -340,7 +344,9 @@ def param_grad(kernel_type: str, x1: Tensor, x2: Tensor, left: Tensor, right: Te
     ``out`` (optional) is a contiguous fp32 tensor [..., P] to write into.  With
     ``static_scratch`` the call goes to km_param_grad_static, which uses the library's per-GPU
     static scratch instead of a workspace allocated here (together with ``out`` the call then
-    allocates nothing; calls that overlap on one GPU must not both use it)."""
+    allocates nothing).  Every GPU has one such array: a call on another stream than the last
+    one is ordered behind it with an event; calls issued from several host threads at once, or
+    through the C ABI directly, must be kept apart by the caller."""
     tensors = (x1, x2, left, right, params, start, end)
     key = _signature("param_grad", kernel_type, tensors)
     prepared = _PREPARED.get(key)
@@ -380,7 +386,16 @@ def param_grad(kernel_type: str, x1: Tensor, x2: Tensor, left: Tensor, right: Te
     out_ptr = out.data_ptr() if out.numel() > 0 else None
     if static_scratch:
         with _on_device(device):
+            stream = torch.cuda.current_stream(device)
+            last = _STATIC_SCRATCH_USE.get(device.index)
+            if last is not None and last[0] != stream.cuda_stream:
+                # The GPU's one scratch array was last used on another stream: order this call
+                # behind that one (calls from several host threads remain the caller's business).
+                stream.wait_event(last[1])
             status = lib.km_param_grad_static(*head, *call_args, out_ptr, _stream(device))
+            event = last[1] if last is not None else torch.cuda.Event()
+            event.record(stream)
+            _STATIC_SCRATCH_USE[device.index] = (stream.cuda_stream, event)
     else:
         workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=device)
         with _on_device(device):

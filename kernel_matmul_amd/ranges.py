@@ -33,7 +33,7 @@ def make_ranges(
     *,
     block_size: int = _BLOCK_SIZE,
     align: bool = False,
-    check_sorted: bool = False,
+    check_sorted: bool = True,
 ) -> tuple[Tensor, Tensor]:
     """Compute the sparsity pattern for a cutoff distance.
 
@@ -50,8 +50,11 @@ def make_ranges(
         block_size: rows per block.
         align: restrict start/end to multiples of ``block_size`` (or ``n2``) so that the
             pattern can be transposed exactly.
-        check_sorted: verify GPU inputs (one host synchronisation) and run unsorted ones
-            through the host scan, so that the result never depends on the tensors' device.
+        check_sorted: verify GPU inputs (one host synchronisation, which the reference's
+            device-to-host copy of every input implies as well) and run unsorted ones through the
+            host scan, so that the result never depends on the tensors' device.  Callers that
+            guarantee sorted input and must not synchronise (stream capture, tight loops) pass
+            ``False``: the device builders then run unconditionally.
 
     Returns:
         ``(start, end)``, int32 tensors of shape ``(batch..., ceil(n1 / block_size))`` on

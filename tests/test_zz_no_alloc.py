@@ -101,3 +101,23 @@ def test_python_binding_without_allocation():
     got = _native.param_grad("spectral", t["x"], t["x"], t["left"], t["right"], t["params"], t["start"], t["end"],
                              out=out, static_scratch=True)
     assert got is out and torch.equal(out, expected)
+
+
+def test_python_binding_orders_static_scratch_calls_across_streams():
+    """Two streams in turn: the binding orders each call behind the last one on the GPU's one
+    scratch array, so both results equal the workspace entry point's."""
+    device = torch.device("cuda:0")
+    a = _problem("spectral", 20_000, 3, 4, seed=45)
+    b = _problem("rbf", 6_000, 2, 3, seed=46)
+    expected = [_native.param_grad(kt, t["x"], t["x"], t["left"], t["right"], t["params"], t["start"], t["end"])
+                for kt, t in (("spectral", a), ("rbf", b))]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(device=device), torch.cuda.Stream(device=device)]
+    outs = [torch.empty_like(e) for e in expected]
+    for _ in range(3):
+        for (kt, t), stream, out in zip((("spectral", a), ("rbf", b)), streams, outs):
+            with torch.cuda.stream(stream):
+                _native.param_grad(kt, t["x"], t["x"], t["left"], t["right"], t["params"], t["start"], t["end"],
+                                   out=out, static_scratch=True)
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0], expected[0]) and torch.equal(outs[1], expected[1])
