@@ -190,12 +190,22 @@ static int make_plan(const MatmulProblem& p, const km_launch_options* opt, Matmu
     const bool two_per_simd = (variant == KM_VARIANT_MFMA_F16_DIRECT && G * R >= 16) ||
                               (variant == KM_VARIANT_MFMA_F16 && table && G == 2);
     const long long wave_target = two_per_simd ? 2 * TARGET_WAVES : TARGET_WAVES;
+    // Table kernel, 128-row items, at least 1.4 items per SIMD: the grouped launch below (one item
+    // per wavefront, the remainder split by columns) rather than column shares for every item.
+    // Measured (spectral, k = 16): n = 1e5, batch 2 (196 items per XCD) 32.9 against 37.5 us, batch 4
+    // (391) 60.3 against 64.1 us; n = 20000, batch 12 (236) 42.3 against 51.0 us; batch 8 (157, below
+    // the bound) 36.9 against 36.6 us.
+    const long long per_xcd_128 = (row_blocks * p.num_batches + KM_NUM_XCD - 1) / KM_NUM_XCD;
+    const bool grouped_128 = table && G == 1 && R == 8 && per_xcd_128 >= 128 + 48 &&
+                             !(opt && (opt->col_splits != 0 || opt->reserved == 1));
     int S = 1;
     if (opt && opt->col_splits != 0) {
         S = opt->col_splits;
         if (S < 1 || S > 8) {
             return fail(KM_ERR_INVALID_ARGUMENT, "km_matmul: col_splits must be 1 to 8");
         }
+    } else if (grouped_128) {
+        S = 1;
     } else if (table && !two_per_simd) {
         // Table kernels: the share count that leaves the fullest SIMD the least work,
         // ceil(wavefronts / 1024) pieces of 1 / S of an item at 8 % of overhead per doubling
@@ -239,6 +249,10 @@ static int make_plan(const MatmulProblem& p, const km_launch_options* opt, Matmu
     // 751 against 773 us); more than a third of a round of wavefronts (128 items) gains nothing.
     if (table && G == 1 && R == 8 && S == 1 && plan->tail_balance && plan->group_tail < 0) {
         const long long per_xcd = (row_blocks * p.num_batches + KM_NUM_XCD - 1) / KM_NUM_XCD;
+        if (per_xcd >= 128 + 48 && per_xcd < 2 * 128) {
+            // one item per SIMD unsplit, everything beyond it split
+            plan->group_tail = per_xcd - 128;
+        }
         if (per_xcd >= 2 * 128) {
             plan->group_tail = per_xcd / 7 < 128 ? per_xcd / 7 : 128;
             if (variant == KM_VARIANT_MFMA_F32) {

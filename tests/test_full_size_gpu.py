@@ -207,6 +207,35 @@ def test_forward_grouped_launch_against_oracle(name, group_tail, halves, rows):
     assert np.all(err <= 1e-5 + 1e-4 * np.abs(expected)), (name, group_tail, halves, err.max())
 
 
+@pytest.mark.parametrize("rows_per_wave", [None, 64])
+def test_forward_grouped_launches_with_a_batch_shape_that_does_not_collapse(rows_per_wave):
+    """The grouped launches (the launch table's choice at this size, and the 64-row one) with two
+    batch dimensions whose strides do not merge (rhs is a slice of a larger tensor): the kernels'
+    general batch addressing instead of the one-stride short cut, every element against the
+    banded oracle."""
+    kernel, n, batch, k, a, h = _build("c3")
+    device = a["x"].device
+    g = torch.Generator().manual_seed(9)
+    big = torch.randn(2, 3, n, k, generator=g).to(device)
+    rhs = big[:, :2]                                   # [2, 2, n, k], batch strides (3nk, nk)
+    params = torch.stack([a["params"], a["params"].flip(0) * 1.1], dim=0)   # [2, 2, 3]
+    rows = a["start"].shape[-1]
+    expand = lambda t, *tail: t.expand(2, 2, *tail)
+    op_args = (expand(a["x"][0], n), expand(a["x"][0], n), rhs, params,
+               expand(a["start"][0], rows), expand(a["end"][0], rows))
+    defines = MatmulSingleConfiguration(kernel).make_config(op_args)
+    if rows_per_wave:
+        defines["MATMUL_ROWS_PER_WAVE"] = rows_per_wave
+        defines["MATMUL_GROUP_TAIL"] = 7
+    op = load_native("matmul", defines)
+    assert ("grouped64" if rows_per_wave else "grouped<") in op.describe(*op_args)
+    out = op.call(*op_args).cpu().double().numpy().reshape(4, n, k)
+    h4 = dict(h, params=params.cpu().numpy().reshape(4, 3))
+    expected = _banded_matmul_oracle(kernel, h4, rhs.cpu().numpy().reshape(4, n, k))
+    err = np.abs(out - expected)
+    assert np.all(err <= 1e-5 + 1e-4 * np.abs(expected)), err.max()
+
+
 def test_split_fp16_error_against_fp32_mfma_on_headline():
     """How much accuracy the split-fp16 contraction (the default) trades against the fp32 MFMA
     contraction, over the full headline output, each against the float64 oracle.  Both must
