@@ -42,6 +42,11 @@ def _lomb_scargle_power(t, y, f_min: float, df: float, num_freqs: int, work_elem
     .score_frequency_grid(f_min, df, num_freqs)`` returns (the reference's call,
     kernel_matmul/util.py:106-108), here from the exact trigonometric sums in float64 instead of
     gatspy's FFT extirpolation.  Runs on the tensors' device, a block of frequencies at a time.
+
+    Cost: O(n * num_freqs) float64 sine / cosine pairs (about 1e11 at the caller's own limits of
+    1e6 frequencies and n ~ 1e5 points) where gatspy's approximation is O(n log n); agreement with
+    gatspy's numbers is not checked anywhere (the package is not available to the tests): the
+    contract is the least-squares definition above, which the tests check directly.
     """
     import torch
 
