@@ -644,18 +644,49 @@ struct ReduceArgs {
     float* grad;  // [num_batches][P]
 };
 
+#define KM_REDUCE_THREADS 1024
+
+// One workgroup per batch item.  Every thread adds its rows (one 16-byte load each, several in
+// flight) in fp64, then a fixed tree over the workgroup: the order of the additions depends on
+// the row count alone, so results are reproducible.
 template <int KT>
-__global__ void __launch_bounds__(256) param_grad_reduce(const ReduceArgs a) {
+__global__ void __launch_bounds__(KM_REDUCE_THREADS) param_grad_reduce(const ReduceArgs a) {
     constexpr int P = KernelTraits<KT>::P;
-    __shared__ double sh[KM_MAX_PARAMS][256];
+    static_assert(KM_MAX_PARAMS == 4, "one float4 per partial row");
+    __shared__ double sh[KM_MAX_PARAMS][KM_REDUCE_THREADS];
     const long long b = blockIdx.x;
-    const float* __restrict__ rows = a.partials + b * a.partial_rows * KM_MAX_PARAMS;
+    const float* __restrict__ base = a.partials + b * a.partial_rows * KM_MAX_PARAMS;
+    // (a workspace that is not 16-byte aligned is read one float at a time)
+    const bool aligned = ((unsigned long long)base & 15ull) == 0;
+    auto load_row = [&](long long r) -> float4v {
+        if (aligned) {
+            return ((const float4v*)base)[r];
+        }
+        const float* q = base + r * KM_MAX_PARAMS;
+        return (float4v){q[0], q[1], q[2], q[3]};
+    };
 
     double sum[KM_MAX_PARAMS] = {0.0, 0.0, 0.0, 0.0};
-    for (long long i = threadIdx.x; i < a.partial_rows; i += 256) {
+    long long i = threadIdx.x;
+    for (; i + 3 * KM_REDUCE_THREADS < a.partial_rows; i += 4 * KM_REDUCE_THREADS) {
+        float4v v[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            v[u] = load_row(i + u * KM_REDUCE_THREADS);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+#pragma unroll
+            for (int p = 0; p < KM_MAX_PARAMS; p++) {
+                sum[p] += (double)v[u][p];
+            }
+        }
+    }
+    for (; i < a.partial_rows; i += KM_REDUCE_THREADS) {
+        const float4v v = load_row(i);
 #pragma unroll
         for (int p = 0; p < KM_MAX_PARAMS; p++) {
-            sum[p] += (double)rows[i * KM_MAX_PARAMS + p];
+            sum[p] += (double)v[p];
         }
     }
 #pragma unroll
@@ -663,7 +694,7 @@ __global__ void __launch_bounds__(256) param_grad_reduce(const ReduceArgs a) {
         sh[p][threadIdx.x] = sum[p];
     }
     __syncthreads();
-    for (int half = 128; half >= 1; half >>= 1) {
+    for (int half = KM_REDUCE_THREADS / 2; half >= 1; half >>= 1) {
         if ((int)threadIdx.x < half) {
 #pragma unroll
             for (int p = 0; p < KM_MAX_PARAMS; p++) {
@@ -807,13 +838,13 @@ hipError_t launch_param_grad_reduce(int kernel_type, const BatchShape& batch, lo
     const unsigned rgrid = (unsigned)num_batches;
     switch (kernel_type) {
         case KM_KERNEL_RBF:
-            hipLaunchKernelGGL((param_grad_reduce<KM_KERNEL_RBF>), dim3(rgrid), dim3(256), 0, stream, ra);
+            hipLaunchKernelGGL((param_grad_reduce<KM_KERNEL_RBF>), dim3(rgrid), dim3(KM_REDUCE_THREADS), 0, stream, ra);
             break;
         case KM_KERNEL_SPECTRAL:
-            hipLaunchKernelGGL((param_grad_reduce<KM_KERNEL_SPECTRAL>), dim3(rgrid), dim3(256), 0, stream, ra);
+            hipLaunchKernelGGL((param_grad_reduce<KM_KERNEL_SPECTRAL>), dim3(rgrid), dim3(KM_REDUCE_THREADS), 0, stream, ra);
             break;
         default:
-            hipLaunchKernelGGL((param_grad_reduce<KM_KERNEL_LOCALLY_PERIODIC>), dim3(rgrid), dim3(256), 0, stream, ra);
+            hipLaunchKernelGGL((param_grad_reduce<KM_KERNEL_LOCALLY_PERIODIC>), dim3(rgrid), dim3(KM_REDUCE_THREADS), 0, stream, ra);
             break;
     }
     return hipGetLastError();
