@@ -254,6 +254,54 @@ class Prepared:
         }
 
 
+def time_index_and_ranges(device, steps=50):
+    """The rest of benchmark configuration 5: kernel rows at 4096 random (batch, row, column) indices
+    and the symmetric range computation at n = 10^6, both on the GPU.  Latency-bound operations:
+    reported as time per call only."""
+    import torch
+
+    from kernel_matmul_amd.compile import load_native
+    from kernel_matmul_amd.configurations import IndexConfiguration
+    from kernel_matmul_amd.ranges import make_ranges
+
+    w, x_cpu, params_cpu, _, cutoff = make_workload("c5")
+    n, batch = w["n"], w["batch"]
+    x = x_cpu.to(device)
+    make_ranges(cutoff, x, check_sorted=False)
+    torch.cuda.synchronize()
+
+    def timed(call):
+        for _ in range(5):
+            call()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            call()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / steps
+
+    ranges_ms = timed(lambda: make_ranges(cutoff, x, check_sorted=False))
+    start, end = make_ranges(cutoff, x, check_sorted=False)
+    g = torch.Generator().manual_seed(w["seed"] + 70)
+    rows = torch.randint(0, n, (4096,), generator=g)
+    cols = torch.clamp(rows + torch.randint(-600, 600, (4096,), generator=g), 0, n - 1)
+    bi = torch.randint(0, batch, (4096,), generator=g)
+    to = lambda t: t.to(torch.int32).to(device)
+    blocks = start.shape[-1]
+    args = (x.expand(batch, n), x.expand(batch, n), params_cpu.to(device), start.expand(batch, blocks),
+            end.expand(batch, blocks), (to(bi),), to(rows), to(cols))
+    op = load_native("index", IndexConfiguration(w["kernel"]).make_config(args))
+    index_ms = timed(lambda: op.call(*args))
+    return {
+        "workload": "spectral, n=1000000, batch=8: index lookup of 4096 random (batch, row, column) entries; "
+                    "symmetric ranges of all 7813 row blocks on the GPU",
+        "index_ms_per_call": index_ms,
+        "ranges_ms_per_call": ranges_ms,
+        "note": "latency-bound operations, wall time per call from Python (launch and argument marshalling "
+                "included); no roofline fraction is meaningful here",
+    }
+
+
 def full_output_fp64(p: Prepared):
     """float64 K @ rhs over the whole pattern of a forward workload, one row block at a time."""
     import numpy as np
@@ -440,6 +488,7 @@ def main() -> int:
             configs[name] = run.summary(steps=20 if name != "c5" else 10, warmup=3)
             del run
             torch.cuda.empty_cache()
+        configs["c5_index_and_ranges"] = time_index_and_ranges(device)
         result["configs"] = configs
 
     if not args.no_cpu_baseline and not main_run.is_grad:
