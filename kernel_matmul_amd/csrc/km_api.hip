@@ -446,8 +446,8 @@ int km_matmul(int kernel_type, int batch_rank, const int64_t* batch_sizes, int64
         KM_REQUIRE_PTR(op, rhs);
     }
 
-    // The kernels address x2 / rhs as a 64-bit base plus a 32-bit lane offset of up to 24 rows
-    // and 64 columns.
+    // The kernels address x2 / rhs as a 64-bit wave-uniform base plus 32-bit byte offsets that
+    // span up to 60 rows and 63 columns of rhs: (60 + 63) * 4 * 2^22 stays below 2^32.
     {
         const int64_t x2_s = x2_strides[batch_rank];
         const int64_t r_s0 = rhs_strides[batch_rank];
@@ -455,8 +455,8 @@ int km_matmul(int kernel_type, int batch_rank, const int64_t* batch_sizes, int64
         if (x2_s < 0 || r_s0 < 0 || r_s1 < 0 || x1_strides[batch_rank] < 0) {
             return fail(KM_ERR_UNSUPPORTED, "%s: negative strides are not supported", op);
         }
-        if (x2_s > (1 << 24) || r_s0 > (1 << 24) || r_s1 > (1 << 24)) {
-            return fail(KM_ERR_UNSUPPORTED, "%s: inner strides above 2^24 elements are not supported", op);
+        if (x2_s > (1 << 22) || r_s0 > (1 << 22) || r_s1 > (1 << 22)) {
+            return fail(KM_ERR_UNSUPPORTED, "%s: inner strides above 2^22 elements are not supported", op);
         }
     }
 

@@ -295,6 +295,29 @@ __device__ __forceinline__ void kernel_pair_f16(float x1, float x2a, float x2b, 
 // Full steps use a wave-uniform base (scalar registers) plus a loop-invariant 32-bit lane
 // offset; the partial last step clamps the column to the range and zeroes the rhs operand of
 // columns past it.
+// Element at a wave-uniform base plus a per-lane offset in BYTES (32 bits).
+__device__ __forceinline__ float load_at(const float* uniform_base, unsigned lane_bytes) {
+    return *(const float*)((const char*)uniform_base + lane_bytes);
+}
+
+// The same through a buffer resource: base and a wave-uniform byte offset in scalar registers,
+// the lane's byte offset in one vector register - no 64-bit vector arithmetic per load (the
+// compiler forms global addresses with a v_lshl_add_u64 each otherwise).  Raw resource over the
+// whole 32-bit offset range: no bounds clamp, offsets stay below 2^32 by the stride limits the
+// entry point checks.
+typedef __amdgpu_buffer_rsrc_t buffer_rsrc;
+__device__ __forceinline__ buffer_rsrc uniform_buffer(const float* uniform_base) {
+    // The base is the same in every lane; reading it from the first lane tells the compiler so
+    // (a resource it takes for divergent is looped over its distinct values around every load).
+    const unsigned long long bits = (unsigned long long)uniform_base;
+    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)bits);
+    const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(bits >> 32));
+    return __builtin_amdgcn_make_buffer_rsrc((void*)(((unsigned long long)hi << 32) | lo), 0, -1, 0x00020000);
+}
+__device__ __forceinline__ float buffer_at(buffer_rsrc rsrc, unsigned lane_bytes, unsigned uniform_bytes) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)lane_bytes, (int)uniform_bytes, 0));
+}
+
 template <int G>
 __device__ __forceinline__ void f16_load(const FwdArgs& a, const WaveView& w, int c0, int col_end,
                                          int kk, unsigned x2_lane, const unsigned (&rhs_lane)[G],
@@ -304,10 +327,10 @@ __device__ __forceinline__ void f16_load(const FwdArgs& a, const WaveView& w, in
         const float* ru = w.rhs + (long long)c0 * a.rhs_s0;
 #pragma unroll
         for (int t = 0; t < 8; t++) {
-            x2v[t] = (x2u + t * a.x2_s)[x2_lane];
+            x2v[t] = load_at(x2u + t * a.x2_s, x2_lane);
 #pragma unroll
             for (int g = 0; g < G; g++) {
-                raw[g][t] = (ru + t * a.rhs_s0)[rhs_lane[g]];
+                raw[g][t] = load_at(ru + t * a.rhs_s0, rhs_lane[g]);
             }
         }
     } else {
@@ -318,7 +341,7 @@ __device__ __forceinline__ void f16_load(const FwdArgs& a, const WaveView& w, in
             x2v[t] = w.x2[(long long)colc * a.x2_s];
 #pragma unroll
             for (int g = 0; g < G; g++) {
-                const float v = w.rhs[(long long)colc * a.rhs_s0 + (rhs_lane[g] - (unsigned)(8 * kk * a.rhs_s0))];
+                const float v = load_at(w.rhs + (long long)colc * a.rhs_s0, rhs_lane[g] - 4u * (unsigned)(8 * kk * a.rhs_s0));
                 raw[g][t] = col < col_end ? v : 0.0f;
             }
         }
@@ -540,19 +563,19 @@ __device__ __forceinline__ void fwd_mfma_f16_body(const FwdArgs& a, float* lds, 
 
     // rhs columns past k read a valid column instead and are zeroed through their scale.
     bool colmask[G];
-    unsigned rhs_lane[G];  // element offset of (column 8 kk, rhs column of this lane)
+    unsigned rhs_lane[G];  // byte offset of (column 8 kk, rhs column of this lane)
     int shift[G];
     float scale[G];
 #pragma unroll
     for (int g = 0; g < G; g++) {
         const int c = kbase + 16 * g + li;
         colmask[g] = c < a.k;
-        rhs_lane[g] = (unsigned)(8 * kk * a.rhs_s0 + (min(c, a.k - 1) - kbase) * a.rhs_s1);
+        rhs_lane[g] = 4u * (unsigned)(8 * kk * a.rhs_s0 + (min(c, a.k - 1) - kbase) * a.rhs_s1);
         // Start far up so that the first non-zero step sets the real scale.
         shift[g] = 100;
         scale[g] = colmask[g] ? __builtin_ldexpf(1.0f, 100) : 0.0f;
     }
-    const unsigned x2_lane = (unsigned)(8 * kk * a.x2_s);
+    const unsigned x2_lane = 4u * (unsigned)(8 * kk * a.x2_s);
 
     float4v acc[R][G];
 #pragma unroll
@@ -661,16 +684,27 @@ __global__ void __launch_bounds__(512) fwd_mfma_f16(const FwdArgs a) {
 #define KM_PHASE_CHUNK 512
 #define KM_PHASE_TABLE_FLOATS (4 * KM_PHASE_CHUNK + KM_PHASE_CHUNK / 8) /* per wavefront */
 
-template <int G>
+template <int G, bool BUFFER>
 __device__ __forceinline__ void rhs_load(const FwdArgs& a, const WaveView& w, int c0, int col_end,
                                          int kk, const unsigned (&rhs_lane)[G], float (&raw)[G][8]) {
     if (c0 + 32 <= col_end) {
-        const float* ru = w.rhs + (long long)c0 * a.rhs_s0;
+        if constexpr (BUFFER) {
+            const buffer_rsrc ru = uniform_buffer(w.rhs + (long long)c0 * a.rhs_s0);
 #pragma unroll
-        for (int t = 0; t < 8; t++) {
+            for (int t = 0; t < 8; t++) {
 #pragma unroll
-            for (int g = 0; g < G; g++) {
-                raw[g][t] = (ru + t * a.rhs_s0)[rhs_lane[g]];
+                for (int g = 0; g < G; g++) {
+                    raw[g][t] = buffer_at(ru, rhs_lane[g], 4u * (unsigned)(t * a.rhs_s0));
+                }
+            }
+        } else {
+            const float* ru = w.rhs + (long long)c0 * a.rhs_s0;
+#pragma unroll
+            for (int t = 0; t < 8; t++) {
+#pragma unroll
+                for (int g = 0; g < G; g++) {
+                    raw[g][t] = load_at(ru + t * a.rhs_s0, rhs_lane[g]);
+                }
             }
         }
     } else {
@@ -680,7 +714,7 @@ __device__ __forceinline__ void rhs_load(const FwdArgs& a, const WaveView& w, in
             const int colc = min(col, col_end - 1);
 #pragma unroll
             for (int g = 0; g < G; g++) {
-                const float v = w.rhs[(long long)colc * a.rhs_s0 + (rhs_lane[g] - (unsigned)(8 * kk * a.rhs_s0))];
+                const float v = load_at(w.rhs + (long long)colc * a.rhs_s0, rhs_lane[g] - 4u * (unsigned)(8 * kk * a.rhs_s0));
                 raw[g][t] = col < col_end ? v : 0.0f;
             }
         }
@@ -744,7 +778,7 @@ __device__ __forceinline__ void fwd_table_body(const FwdArgs& a, float* lds, con
 #pragma unroll
     for (int g = 0; g < G; g++) {
         const int c = kbase + 16 * g + li;
-        rhs_lane[g] = (unsigned)(8 * kk * a.rhs_s0 + (min(c, a.k - 1) - kbase) * a.rhs_s1);
+        rhs_lane[g] = 4u * (unsigned)(8 * kk * a.rhs_s0 + (min(c, a.k - 1) - kbase) * a.rhs_s1);
         colmask[g] = c < a.k;
         shift[g] = F32 ? 0 : 100;
         scale[g] = c < a.k ? __builtin_ldexpf(1.0f, 100) : 0.0f;
@@ -800,7 +834,7 @@ __device__ __forceinline__ void fwd_table_body(const FwdArgs& a, float* lds, con
     auto build = [&](int chunk0, bool allow) -> bool {
         const int chunk_end = min(chunk0 + CH, col_end);
         const int padded = (chunk_end - chunk0 + 31) & ~31;
-        // Strides are below 2^24 elements, so 32 x 32 -> 64 bit products are enough.
+        // Strides are below 2^22 elements, so 32 x 32 -> 64 bit products are enough.
         const float* x2c = w.x2 + (long long)chunk0 * a.x2_s;
         const unsigned x2_stride = (unsigned)a.x2_s;
         const int last = chunk_end - 1 - chunk0;
@@ -880,7 +914,7 @@ __device__ __forceinline__ void fwd_table_body(const FwdArgs& a, float* lds, con
     float raw[G][8];
     auto request_first = [&](int chunk0) {
         if (F32) {
-            rhs_load<G>(a, w, chunk0, min(chunk0 + CH, col_end), kk, rhs_lane, raw);
+            rhs_load<G, !F32>(a, w, chunk0, min(chunk0 + CH, col_end), kk, rhs_lane, raw);
         }
     };
 
@@ -889,7 +923,7 @@ __device__ __forceinline__ void fwd_table_body(const FwdArgs& a, float* lds, con
         constexpr bool SEP = decltype(sep_c)::value;
         const int chunk_end = min(chunk0 + CH, col_end);
         if (!F32) {
-            rhs_load<G>(a, w, chunk0, chunk_end, kk, rhs_lane, raw);
+            rhs_load<G, !F32>(a, w, chunk0, chunk_end, kk, rhs_lane, raw);
         }
         for (int c0 = chunk0; c0 < chunk_end; c0 += 32) {
             const int off = c0 - chunk0 + 8 * kk;
@@ -922,7 +956,7 @@ __device__ __forceinline__ void fwd_table_body(const FwdArgs& a, float* lds, con
                 // The next step's rhs operand is requested before this step is evaluated.
                 float rawn[G][8];
                 if (c0 + 32 < chunk_end) {
-                    rhs_load<G>(a, w, c0 + 32, chunk_end, kk, rhs_lane, rawn);
+                    rhs_load<G, !F32>(a, w, c0 + 32, chunk_end, kk, rhs_lane, rawn);
                 }
                 f32_step<KT, G, R, SEP>(x2v, raw, x1v, kc, acc, ref, cb, sb, row_cos, row_sin);
                 if (c0 + 32 < chunk_end) {
@@ -940,7 +974,7 @@ __device__ __forceinline__ void fwd_table_body(const FwdArgs& a, float* lds, con
                          PAIRCOS && SEP>(x2v, raw, x1v, kc, colmask, shift, scale, acc, ref, cb, sb, row_phase);
             }
             if (c0 + 32 < chunk_end) {
-                rhs_load<G>(a, w, c0 + 32, chunk_end, kk, rhs_lane, raw);
+                rhs_load<G, !F32>(a, w, c0 + 32, chunk_end, kk, rhs_lane, raw);
             }
         }
         // All reads of the table are done before the next chunk overwrites it.
