@@ -295,29 +295,6 @@ __device__ __forceinline__ void kernel_pair_f16(float x1, float x2a, float x2b, 
 // Full steps use a wave-uniform base (scalar registers) plus a loop-invariant 32-bit lane
 // offset; the partial last step clamps the column to the range and zeroes the rhs operand of
 // columns past it.
-// Element at a wave-uniform base plus a per-lane offset in BYTES (32 bits).
-__device__ __forceinline__ float load_at(const float* uniform_base, unsigned lane_bytes) {
-    return *(const float*)((const char*)uniform_base + lane_bytes);
-}
-
-// The same through a buffer resource: base and a wave-uniform byte offset in scalar registers,
-// the lane's byte offset in one vector register - no 64-bit vector arithmetic per load (the
-// compiler forms global addresses with a v_lshl_add_u64 each otherwise).  Raw resource over the
-// whole 32-bit offset range: no bounds clamp, offsets stay below 2^32 by the stride limits the
-// entry point checks.
-typedef __amdgpu_buffer_rsrc_t buffer_rsrc;
-__device__ __forceinline__ buffer_rsrc uniform_buffer(const float* uniform_base) {
-    // The base is the same in every lane; reading it from the first lane tells the compiler so
-    // (a resource it takes for divergent is looped over its distinct values around every load).
-    const unsigned long long bits = (unsigned long long)uniform_base;
-    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)bits);
-    const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(bits >> 32));
-    return __builtin_amdgcn_make_buffer_rsrc((void*)(((unsigned long long)hi << 32) | lo), 0, -1, 0x00020000);
-}
-__device__ __forceinline__ float buffer_at(buffer_rsrc rsrc, unsigned lane_bytes, unsigned uniform_bytes) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)lane_bytes, (int)uniform_bytes, 0));
-}
-
 template <int G>
 __device__ __forceinline__ void f16_load(const FwdArgs& a, const WaveView& w, int c0, int col_end,
                                          int kk, unsigned x2_lane, const unsigned (&rhs_lane)[G],
