@@ -120,6 +120,8 @@ int km_make_ranges_symmetric_device(const float* x, int64_t num_batch, int64_t n
  * native/matmul/matmul.cu:160-203).
  *   x1[batch..., m], x2[batch..., n], rhs[batch..., n, k], params[batch..., P],
  *   start/end[batch..., ceil(m/128)], out[batch..., m, k] contiguous.
+ * The strides of x1, x2 and rhs along their own dimensions must not be negative, and those of x2
+ * and rhs at most 2^22 elements (KM_ERR_UNSUPPORTED otherwise); batch strides are free.
  * ---------------------------------------------------------------------------------- */
 int km_matmul(int kernel_type, int batch_rank, const int64_t* batch_sizes, int64_t m, int64_t n,
               int64_t k, const float* x1, const int64_t* x1_strides, const float* x2,
