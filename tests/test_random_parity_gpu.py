@@ -2,8 +2,10 @@
 
 Shapes, batch shapes, coordinate units and offsets (the regimes that decide between the separable
 and the direct evaluation), lengthscales, frequencies, signs of the outputscale, cutoffs, sorted
-and unsorted coordinates with arbitrary ranges, rhs magnitudes, contraction variants and launch
-shapes are drawn at random; every case is compared element by element.
+and unsorted coordinates with arbitrary ranges, rhs magnitudes, contraction variants, launch
+shapes and memory layouts (a quarter of the tensors are handed over as strided views: transposed,
+cut out of a wider tensor, or every second element) are drawn at random; every case is compared
+element by element.
 
 Tolerance of the forward result, per element: 1e-5 max|rhs| + 1e-4 |expected| + 2e-6 |K| @ |rhs|
 (fp32 evaluation and accumulation), plus, for the oscillating kernels, the fp32 rounding of the
@@ -24,6 +26,7 @@ from kernel_matmul_amd.compile import load_native
 from kernel_matmul_amd.configurations import BilinearDerivativeConfiguration, MatmulSingleConfiguration
 from kernel_matmul_amd.ranges import make_ranges
 from oracle import kernels as oracle
+from tests.test_strided_inputs_gpu import column_major, interleaved, padded
 
 pytestmark = pytest.mark.gpu
 
@@ -75,6 +78,19 @@ def _draw(rng):
                 rows_per_wave=rows_per_wave, splits=splits, left=left, right=right)
 
 
+def _on_device(d, keys, device, layouts):
+    """The tensors of a case on the GPU, some of them as strided views of the same values (drawn
+    from a generator of its own, so that the cases themselves do not depend on it)."""
+    out = []
+    for key in keys:
+        t = d[key].to(device)
+        if t.numel() > 0 and layouts.random() < 0.25:
+            matrix = key in ("rhs", "left", "right")
+            t = layouts.choice([column_major, padded, interleaved] if matrix else [padded, interleaved])(t)
+        out.append(t)
+    return tuple(out)
+
+
 @pytest.mark.parametrize("seed", [1, 2, 3])
 def test_random_cases_against_oracle(seed):
     rng = random.Random(seed)
@@ -85,7 +101,8 @@ def test_random_cases_against_oracle(seed):
         kt = d["kt"]
         what = (seed, case, kt, tuple(d["x1"].shape), tuple(d["rhs"].shape), d["variant"], d["rows_per_wave"],
                 d["splits"])
-        args = tuple(d[key].to(device) for key in ("x1", "x2", "rhs", "params", "start", "end"))
+        layouts = random.Random(7919 * seed + case)
+        args = _on_device(d, ("x1", "x2", "rhs", "params", "start", "end"), device, layouts)
         defines = MatmulSingleConfiguration(kt).make_config(args)
         if d["variant"]:
             defines["MATMUL_VARIANT"] = d["variant"]
@@ -110,7 +127,7 @@ def test_random_cases_against_oracle(seed):
         assert np.all(np.isfinite(out)), what
         assert np.all(np.abs(out - expected) <= tol), (what, float(np.max(np.abs(out - expected) / tol)))
 
-        gargs = tuple(d[key].to(device) for key in ("x1", "x2", "left", "right", "params", "start", "end"))
+        gargs = _on_device(d, ("x1", "x2", "left", "right", "params", "start", "end"), device, layouts)
         got = load_native("bilinear_derivative", BilinearDerivativeConfiguration(kt).make_config(gargs)).call(*gargs)
         got = got.cpu().double().numpy()
         left, right = d["left"].numpy(), d["right"].numpy()
