@@ -451,6 +451,10 @@ def main() -> int:
             "pipe": pipe_of(main_run.kernel),
             "valu_busy": VALU_BUSY["headline"][0] if default_run else None,
             "valu_busy_source": VALU_BUSY["headline"][1] if default_run else None,
+            # what the launched kernel executes per wavefront-wide group of 64 pairs (SQ_INSTS_VALU and
+            # SQ_INSTS_MFMA of the same counter runs over the 5.14 M groups of a launch)
+            "executed_per_64_pairs": {"valu_instructions": 8.1, "mfma_f32_16x16x32_f16": 0.75}
+                                     if default_run else None,
             "achieved_is": "nominal flops per pair (8 + 2k: direct evaluation, fp32 contraction) x pairs / kernel "
                            "time; the kernel launched executes fewer VALU operations per pair (separable exponent, "
                            "tabulated phases) and contracts on the matrix pipe named in `pipe`",
