@@ -30,6 +30,7 @@ struct GradArgs {
     long long num_batches;
     long long total_items;  // row blocks * col splits * batches
     long long items_per_xcd;
+    long long partial_rows;  // total_items / num_batches
     int m, n, c;
     int col_splits;
     const float* x1;
@@ -48,7 +49,15 @@ struct GradArgs {
 // [col_begin, col_end), sums written to `prow` (KM_MAX_PARAMS floats).
 // TL > 0: the vector width c is at most 4*TL and the left operand stays in registers.
 // TL == 0: any c; the left operand is re-read (from L1/L2) for every column chunk.
-template <int KT, int TL, int R>
+//
+// FAST: every inner stride is non-negative and at most KM_GRAD_FAST_STRIDE elements (the host
+// checks).  Addresses are then a wave-uniform 64-bit base, advanced on the scalar unit, plus a
+// loop-invariant 32-bit lane offset formed once with 24-bit multiplies; the general form pays
+// a 64-bit vector multiplication (four quarter-rate instructions) per load, which for a short
+// column share is a third of the wavefront's issue time (48 row operands against three chunks).
+#define KM_GRAD_FAST_STRIDE (1 << 21)
+
+template <int KT, int TL, int R, bool FAST = false>
 __device__ __forceinline__ void pairwise_item(const GradArgs& a, const float* __restrict__ x1,
                                               const float* __restrict__ x2, const float* __restrict__ left,
                                               const float* __restrict__ right, const KernelConsts& kc,
@@ -58,30 +67,91 @@ __device__ __forceinline__ void pairwise_item(const GradArgs& a, const float* __
     const int li = lane & 15;
     const int kk = lane >> 4;
 
-    // x1 for the 4 rows per row group this lane owns in the D layout.
-    float x1q[R][4];
-#pragma unroll
-    for (int r = 0; r < R; r++) {
-#pragma unroll
-        for (int v = 0; v < 4; v++) {
-            const int row = min(row0 + 16 * r + 4 * kk + v, a.m - 1);
-            x1q[r][v] = x1[(long long)row * a.x1_s];
-        }
-    }
-
-    // Left operand (A layout): row = row0 + 16 r + li, vector column = 4 t + kk.
+    // x1 for the 4 rows per row group this lane owns in the D layout, and the left operand
+    // (A layout): row = row0 + 16 r + li, vector column = 4 t + kk.
     constexpr int TLR = TL > 0 ? TL : 1;
+    float x1q[R][4];
     float lreg[R][TLR];
-    if (TL > 0) {
+    // FAST: lane offsets (bytes) of the vector columns 4 t + kk, clamped into the row, and whether
+    // the column exists.
+    unsigned left_col[TLR], right_col[TLR];
+    bool col_used[TLR];
+    if (FAST) {
+        const unsigned x1_s = (unsigned)a.x1_s, l0 = (unsigned)a.left_s0, l1 = (unsigned)a.left_s1;
+        const unsigned r1 = (unsigned)a.right_s1;
 #pragma unroll
-        for (int r = 0; r < R; r++) {
-            const int row = row0 + 16 * r + li;
+        for (int t = 0; t < TLR; t++) {
+            const unsigned cc = (unsigned)min(4 * t + kk, a.c - 1);
+            col_used[t] = 4 * t + kk < a.c;
+            left_col[t] = 4u * __umul24(cc, l1);
+            right_col[t] = 4u * __umul24(cc, r1);
+        }
+        // (buffer loads: base and row offset in scalar registers, see uniform_buffer)
+        const buffer_rsrc x1_rows = uniform_buffer(x1 + (long long)row0 * a.x1_s);
+        const buffer_rsrc left_rows = uniform_buffer(left + (long long)row0 * a.left_s0);
+        if (row0 + 16 * R <= a.m) {
+            const unsigned x1_lane = 4u * __umul24(4u * (unsigned)kk, x1_s);
+            const unsigned left_lane = 4u * __umul24((unsigned)li, l0);
+            unsigned left_lane_col[TLR];
 #pragma unroll
             for (int t = 0; t < TLR; t++) {
-                const int cc = 4 * t + kk;
-                lreg[r][t] = (row < a.m && cc < a.c)
-                                 ? left[(long long)row * a.left_s0 + (long long)cc * a.left_s1]
-                                 : 0.0f;
+                left_lane_col[t] = left_lane + left_col[t];
+            }
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    x1q[r][v] = buffer_at(x1_rows, x1_lane, 4u * (unsigned)(16 * r + v) * x1_s);
+                }
+                if (TL > 0) {
+#pragma unroll
+                    for (int t = 0; t < TLR; t++) {
+                        const float value = buffer_at(left_rows, left_lane_col[t], 4u * (unsigned)(16 * r) * l0);
+                        lreg[r][t] = col_used[t] ? value : 0.0f;
+                    }
+                }
+            }
+        } else {
+            // The last row block: rows past m read row m - 1 (x1) or count as zero (left).
+            const int last = a.m - 1 - row0;
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const unsigned rel = (unsigned)min(16 * r + 4 * kk + v, last);
+                    x1q[r][v] = buffer_at(x1_rows, 4u * __umul24(rel, x1_s), 0u);
+                }
+                if (TL > 0) {
+                    const int rel = 16 * r + li;
+                    const unsigned row_off = 4u * __umul24((unsigned)min(rel, last), l0);
+#pragma unroll
+                    for (int t = 0; t < TLR; t++) {
+                        const float value = buffer_at(left_rows, row_off + left_col[t], 0u);
+                        lreg[r][t] = (rel <= last && col_used[t]) ? value : 0.0f;
+                    }
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const int row = min(row0 + 16 * r + 4 * kk + v, a.m - 1);
+                x1q[r][v] = x1[(long long)row * a.x1_s];
+            }
+        }
+        if (TL > 0) {
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                const int row = row0 + 16 * r + li;
+#pragma unroll
+                for (int t = 0; t < TLR; t++) {
+                    const int cc = 4 * t + kk;
+                    lreg[r][t] = (row < a.m && cc < a.c)
+                                     ? left[(long long)row * a.left_s0 + (long long)cc * a.left_s1]
+                                     : 0.0f;
+                }
             }
         }
     }
@@ -91,9 +161,41 @@ __device__ __forceinline__ void pairwise_item(const GradArgs& a, const float* __
     // Operands of a chunk of 16 columns: x2 of column n0 + li and, with the left operand in
     // registers, the right operand's values (column n0 + li, vector column 4 t + kk), zero outside
     // the range.  They are requested one chunk ahead.
+    const unsigned x2_lane = FAST ? 4u * __umul24((unsigned)li, (unsigned)a.x2_s) : 0u;
+    unsigned right_lane_col[TLR];
+#pragma unroll
+    for (int t = 0; t < TLR; t++) {
+        right_lane_col[t] = FAST ? 4u * __umul24((unsigned)li, (unsigned)a.right_s0) + right_col[t] : 0u;
+    }
     auto load_chunk = [&](int n0, float* x2v, float (&rv)[TLR]) {
         const int col = n0 + li;
         const int col_c = min(col, col_end - 1);
+        if (FAST) {
+            const buffer_rsrc x2_cols = uniform_buffer(x2 + (long long)n0 * a.x2_s);
+            const buffer_rsrc right_cols = uniform_buffer(right + (long long)n0 * a.right_s0);
+            // (values of columns past the range or the vector width are zeroed where they are
+            // used, one chunk later: a select here would wait for the load at once)
+            if (n0 + 16 <= col_end) {
+                *x2v = buffer_at(x2_cols, x2_lane, 0u);
+                if (TL > 0) {
+#pragma unroll
+                    for (int t = 0; t < TLR; t++) {
+                        rv[t] = buffer_at(right_cols, right_lane_col[t], 0u);
+                    }
+                }
+            } else {
+                const unsigned rel = (unsigned)(col_c - n0);
+                *x2v = buffer_at(x2_cols, 4u * __umul24(rel, (unsigned)a.x2_s), 0u);
+                if (TL > 0) {
+                    const unsigned col_off = 4u * __umul24(rel, (unsigned)a.right_s0);
+#pragma unroll
+                    for (int t = 0; t < TLR; t++) {
+                        rv[t] = buffer_at(right_cols, col_off + right_col[t], 0u);
+                    }
+                }
+            }
+            return;
+        }
         *x2v = x2[(long long)col_c * a.x2_s];
         if (TL > 0) {
 #pragma unroll
@@ -118,7 +220,7 @@ __device__ __forceinline__ void pairwise_item(const GradArgs& a, const float* __
         float rvs[TLR];
 #pragma unroll
         for (int t = 0; t < TLR; t++) {
-            rvs[t] = rv_next[t];
+            rvs[t] = (!FAST || (col_ok && col_used[t])) ? rv_next[t] : 0.0f;
         }
         if (n0 + 16 < col_end) {
             load_chunk(n0 + 16, &x2_next, rv_next);
@@ -186,15 +288,31 @@ struct GradItem {
     const float* params;
 };
 
+// FAST: all counts are below 2^31 (the host checks): 32-bit divisions.
+template <bool FAST = false>
 __device__ __forceinline__ bool grad_item(const GradArgs& a, int rows_per_item, int col_step, GradItem* g) {
-    const long long item = xcd_item(blockIdx.x, a.items_per_xcd);
-    if (item >= a.total_items) {
-        return false;
+    int split, chunk;
+    if (FAST) {
+        const unsigned item = (blockIdx.x % KM_NUM_XCD) * (unsigned)a.items_per_xcd + blockIdx.x / KM_NUM_XCD;
+        if (item >= (unsigned)a.total_items) {
+            return false;
+        }
+        const unsigned batches = (unsigned)a.num_batches;
+        const unsigned rest = item / batches;
+        g->b = item - rest * batches;
+        g->rest = rest;
+        chunk = (int)(rest / (unsigned)a.col_splits);
+        split = (int)(rest - (unsigned)chunk * (unsigned)a.col_splits);
+    } else {
+        const long long item = xcd_item(blockIdx.x, a.items_per_xcd);
+        if (item >= a.total_items) {
+            return false;
+        }
+        g->b = item % a.num_batches;
+        g->rest = item / a.num_batches;
+        split = (int)(g->rest % a.col_splits);
+        chunk = (int)(g->rest / a.col_splits);
     }
-    g->b = item % a.num_batches;
-    g->rest = item / a.num_batches;
-    const int split = (int)(g->rest % a.col_splits);
-    const int chunk = (int)(g->rest / a.col_splits);
     const int chunks_per_block = KM_BLOCK_SIZE / rows_per_item;
     const int row_block = chunk / chunks_per_block;
     g->row0 = row_block * KM_BLOCK_SIZE + (chunk % chunks_per_block) * rows_per_item;
@@ -233,16 +351,15 @@ __device__ __forceinline__ bool grad_item(const GradArgs& a, int rows_per_item, 
     return true;
 }
 
-template <int KT, int TL>
+template <int KT, int TL, bool FAST>
 __global__ void __launch_bounds__(64) param_grad_partial(const GradArgs a) {
     GradItem g;
-    if (!grad_item(a, KM_BLOCK_SIZE, 16, &g)) {
+    if (!grad_item<FAST>(a, KM_BLOCK_SIZE, 16, &g)) {
         return;
     }
     const KernelConsts kc = make_consts<KT>(g.params, a.params_s, false);
-    const long long partial_rows = a.total_items / a.num_batches;
-    pairwise_item<KT, TL, 8>(a, g.x1, g.x2, g.left, g.right, kc, g.row0, g.col_begin, g.col_end,
-                             a.partials + (g.b * partial_rows + g.rest) * KM_MAX_PARAMS);
+    pairwise_item<KT, TL, 8, FAST>(a, g.x1, g.x2, g.left, g.right, kc, g.row0, g.col_begin, g.col_end,
+                                   a.partials + (g.b * a.partial_rows + g.rest) * KM_MAX_PARAMS);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -304,8 +421,7 @@ __global__ void __launch_bounds__(64, 2) param_grad_features(const GradArgs a) {
     const int li = lane & 15;
     const int kk = lane >> 4;
     const KernelConsts kc = make_consts<KT>(g.params, a.params_s, false);
-    const long long partial_rows = a.total_items / a.num_batches;
-    float* __restrict__ prow = a.partials + (g.b * partial_rows + g.rest) * KM_MAX_PARAMS;
+    float* __restrict__ prow = a.partials + (g.b * a.partial_rows + g.rest) * KM_MAX_PARAMS;
     const int row0 = g.row0;
     const int col_begin = g.col_begin, col_end = g.col_end;
 
@@ -809,18 +925,38 @@ static hipError_t launch_features(int kernel_type, const FeaturePlan& f, const G
     return launch_features_as<KM_KERNEL_RBF, 2, 8, 4>(a, grid_x, stream);
 }
 
-template <int KT>
-static hipError_t launch_partial(const GradArgs& a, unsigned grid_x, hipStream_t stream) {
+// The short addressing and decode of the pairwise kernel apply when the batch shape has
+// collapsed to at most one dimension, all counts fit 31 bits and the inner strides are small.
+static bool pairwise_fast(const GradArgs& a) {
+    const long long limit = 1ll << 31;
+    const long long strides[6] = {a.x1_s, a.x2_s, a.left_s0, a.left_s1, a.right_s0, a.right_s1};
+    for (long long stride : strides) {
+        if (stride < 0 || stride > KM_GRAD_FAST_STRIDE) {
+            return false;
+        }
+    }
+    return a.batch.rank <= 1 && a.c >= 1 && a.total_items < limit && a.items_per_xcd * KM_NUM_XCD < limit &&
+           a.num_batches < limit;
+}
+
+template <int KT, bool FAST>
+static hipError_t launch_partial_as(const GradArgs& a, unsigned grid_x, hipStream_t stream) {
     if (a.c <= 4) {
-        hipLaunchKernelGGL((param_grad_partial<KT, 1>), dim3(grid_x), dim3(64), 0, stream, a);
+        hipLaunchKernelGGL((param_grad_partial<KT, 1, FAST>), dim3(grid_x), dim3(64), 0, stream, a);
     } else if (a.c <= 8) {
-        hipLaunchKernelGGL((param_grad_partial<KT, 2>), dim3(grid_x), dim3(64), 0, stream, a);
+        hipLaunchKernelGGL((param_grad_partial<KT, 2, FAST>), dim3(grid_x), dim3(64), 0, stream, a);
     } else if (a.c <= 16) {
-        hipLaunchKernelGGL((param_grad_partial<KT, 4>), dim3(grid_x), dim3(64), 0, stream, a);
+        hipLaunchKernelGGL((param_grad_partial<KT, 4, FAST>), dim3(grid_x), dim3(64), 0, stream, a);
     } else {
-        hipLaunchKernelGGL((param_grad_partial<KT, 0>), dim3(grid_x), dim3(64), 0, stream, a);
+        hipLaunchKernelGGL((param_grad_partial<KT, 0, FAST>), dim3(grid_x), dim3(64), 0, stream, a);
     }
     return hipGetLastError();
+}
+
+template <int KT>
+static hipError_t launch_partial(const GradArgs& a, unsigned grid_x, hipStream_t stream) {
+    return pairwise_fast(a) ? launch_partial_as<KT, true>(a, grid_x, stream)
+                            : launch_partial_as<KT, false>(a, grid_x, stream);
 }
 
 hipError_t launch_param_grad_reduce(int kernel_type, const BatchShape& batch, long long num_batches,
@@ -880,6 +1016,7 @@ hipError_t launch_param_grad(const ParamGradProblem& p, hipStream_t stream) {
     a.col_splits = grad_col_splits(chunks * p.num_batches, fplan.GE > 0);
     a.total_items = chunks * a.col_splits * p.num_batches;
     a.items_per_xcd = (a.total_items + KM_NUM_XCD - 1) / KM_NUM_XCD;
+    a.partial_rows = chunks * a.col_splits;
     a.x1 = p.x1;
     a.x2 = p.x2;
     a.left = p.left;
