@@ -65,11 +65,11 @@ VALU_BUSY = {
     "headline_fp32": (0.46, "profiles/fwd_table_f32_grouped_headline_profile.md"),
     "c1": (0.11, "profiles/fwd_table_f16_midsize_c1_c2_c3_profile.md"),
     "c2": (0.46, "profiles/fwd_table_f16_midsize_c1_c2_c3_profile.md"),
-    "c3": (0.51, "profiles/param_grad_partial_c3_and_wide_vectors_profile.md"),
+    "c3": (0.45, "profiles/param_grad_partial_c3_and_wide_vectors_profile.md"),
     "c3_rhs_grad": (0.47, "profiles/fwd_table_f16_midsize_c1_c2_c3_profile.md"),
     "c4": (0.73, "profiles/param_grad_features_c4_profile.md"),
     "c5": (0.95, "profiles/forward_c5_and_reference_recipe_profile.md"),
-    "grad_c8": (0.65, "profiles/param_grad_partial_c3_and_wide_vectors_profile.md"),
+    "grad_c8": (0.62, "profiles/param_grad_partial_c3_and_wide_vectors_profile.md"),
     "ref_example": (0.43, "profiles/forward_c5_and_reference_recipe_profile.md"),
 }
 
