@@ -89,3 +89,25 @@ def test_ranges_of_the_documented_binding(stub):
     start, end = stub["_native"].make_ranges_symmetric(x.to("cuda:0"), 2.5, 128)
     expected_start, expected_end = make_ranges(2.5, x)
     assert start.is_cuda and torch.equal(start.cpu(), expected_start) and torch.equal(end.cpu(), expected_end)
+
+
+def test_usage_example_of_the_readme():
+    """The "Use" block of README.md runs as written; the first row block of its product is checked
+    against the oracle."""
+    text = open(os.path.join(ROOT, "README.md"), encoding="utf-8").read()
+    block = re.search(r"## Use.*?```python\n(.*?)```", text, re.S).group(1)
+    namespace = {}
+    torch.manual_seed(24)
+    exec(compile(block, "README.md", "exec"), namespace)
+    x, params, start, end, y = (namespace[name] for name in ("x", "params", "start", "end", "y"))
+    assert y.shape == (100_000, 16) and bool(torch.isfinite(y).all())
+    # y = K @ rhs with an rhs the block does not keep: linearity pins the operator instead
+    rhs = torch.randn(100_000, 16, device=x.device)
+    product = namespace["K"] @ rhs
+    rows = slice(0, 128)
+    first, last = int(start[0]), int(end[0])
+    expected = oracle.matmul("spectral", x[rows].cpu().numpy(), x[first:last].cpu().numpy(),
+                             rhs[first:last].cpu().numpy(), params.cpu().numpy(),
+                             np.array([0], dtype=np.int32), np.array([last - first], dtype=np.int32))
+    got = product[rows].cpu().double().numpy()
+    assert np.all(np.abs(got - expected) <= ATOL + RTOL * np.abs(expected))
