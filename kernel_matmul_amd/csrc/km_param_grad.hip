@@ -25,8 +25,11 @@
 
 namespace km {
 
+// The first 240 bytes are everything a wavefront of the pairwise kernel reads when the batch
+// shape has collapsed to at most one dimension: contiguous, so that its prologue fetches the
+// argument block with a few wide scalar loads issued together instead of a chain of dependent
+// ones.
 struct GradArgs {
-    BatchShape batch;
     long long num_batches;
     long long total_items;  // row blocks * col splits * batches
     long long items_per_xcd;
@@ -41,8 +44,10 @@ struct GradArgs {
     const int* start;
     const int* end;
     float* partials;  // [num_batches][row_blocks * col_splits][KM_MAX_PARAMS]
-    BatchStrides x1_bs, x2_bs, left_bs, right_bs, params_bs, start_bs, end_bs;
+    long long first_bs[7];  // stride of the first batch dimension of x1, x2, left, right, params, start, end
     long long x1_s, x2_s, left_s0, left_s1, right_s0, right_s1, params_s, start_s, end_s;
+    BatchShape batch;
+    BatchStrides x1_bs, x2_bs, left_bs, right_bs, params_bs, start_bs, end_bs;
 };
 
 // One item of the pairwise form: R groups of 16 rows from row0 against the columns
@@ -318,7 +323,16 @@ __device__ __forceinline__ bool grad_item(const GradArgs& a, int rows_per_item, 
     g->row0 = row_block * KM_BLOCK_SIZE + (chunk % chunks_per_block) * rows_per_item;
 
     long long off_start, off_end;
-    if (a.batch.rank <= 1) {
+    if (FAST) {
+        // (launched for collapsed batch shapes only)
+        g->x1 = a.x1 + g->b * a.first_bs[0];
+        g->x2 = a.x2 + g->b * a.first_bs[1];
+        g->left = a.left + g->b * a.first_bs[2];
+        g->right = a.right + g->b * a.first_bs[3];
+        g->params = a.params + g->b * a.first_bs[4];
+        off_start = g->b * a.first_bs[5];
+        off_end = g->b * a.first_bs[6];
+    } else if (a.batch.rank <= 1) {
         // The usual case after the host has collapsed the batch dimensions: one stride per tensor.
         g->x1 = a.x1 + g->b * a.x1_bs.s[0];
         g->x2 = a.x2 + g->b * a.x2_bs.s[0];
@@ -353,6 +367,18 @@ __device__ __forceinline__ bool grad_item(const GradArgs& a, int rows_per_item, 
 
 template <int KT, int TL, bool FAST>
 __global__ void __launch_bounds__(64) param_grad_partial(const GradArgs a) {
+    if (FAST) {
+        // All of the argument block's hot part is requested here, in one go: left to the
+        // compiler the loads are issued where each value is first used, one round trip to the
+        // scalar cache after the other (six before the first row operand is requested).
+        asm volatile("" ::"s"(a.num_batches), "s"(a.total_items), "s"(a.items_per_xcd), "s"(a.partial_rows),
+                     "s"(a.m), "s"(a.n), "s"(a.c), "s"(a.col_splits), "s"(a.x1), "s"(a.x2), "s"(a.left),
+                     "s"(a.right), "s"(a.params), "s"(a.start), "s"(a.end), "s"(a.partials));
+        asm volatile("" ::"s"(a.first_bs[0]), "s"(a.first_bs[1]), "s"(a.first_bs[2]), "s"(a.first_bs[3]),
+                     "s"(a.first_bs[4]), "s"(a.first_bs[5]), "s"(a.first_bs[6]), "s"(a.x1_s), "s"(a.x2_s),
+                     "s"(a.left_s0), "s"(a.left_s1), "s"(a.right_s0), "s"(a.right_s1), "s"(a.params_s),
+                     "s"(a.start_s), "s"(a.end_s));
+    }
     GradItem g;
     if (!grad_item<FAST>(a, KM_BLOCK_SIZE, 16, &g)) {
         return;
@@ -1017,6 +1043,13 @@ hipError_t launch_param_grad(const ParamGradProblem& p, hipStream_t stream) {
     a.total_items = chunks * a.col_splits * p.num_batches;
     a.items_per_xcd = (a.total_items + KM_NUM_XCD - 1) / KM_NUM_XCD;
     a.partial_rows = chunks * a.col_splits;
+    {
+        const BatchStrides* const all[7] = {&a.x1_bs, &a.x2_bs, &a.left_bs, &a.right_bs,
+                                            &a.params_bs, &a.start_bs, &a.end_bs};
+        for (int i = 0; i < 7; i++) {
+            a.first_bs[i] = a.batch.rank >= 1 ? all[i]->s[0] : 0;
+        }
+    }
     a.x1 = p.x1;
     a.x2 = p.x2;
     a.left = p.left;
